@@ -1,0 +1,279 @@
+"""ctypes binding of ``libilgpu_hip_algorithms.so`` (the C ABI declared in
+``include/ilgpu_hip_algorithms.h``).
+
+Device memory and streams come from torch (plumbing only): a ``DeviceArray``
+is a raw byte tensor on ``cuda:0`` plus the numpy dtype of its elements, so
+every ILGPU element type, including the unsigned ones torch has no arithmetic
+for, can be passed by pointer.
+
+Loading fails loudly when the shared library has not been built; there is no
+fallback implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libilgpu_hip_algorithms.so")
+
+# ilgpu_hip_status
+SUCCESS, ERROR_NULL_VIEW, ERROR_OUT_OF_RANGE, ERROR_NOT_SUPPORTED, \
+    ERROR_UNALIGNED_TEMP, ERROR_RUNTIME = range(6)
+# ilgpu_hip_type
+I8, I16, I32, I64, U8, U16, U32, U64, F16, F32, F64 = range(11)
+# ilgpu_hip_op / scan kind / flags / value source / locator
+OP_ADD, OP_MAX, OP_MIN = 0, 1, 2
+SCAN_INCLUSIVE, SCAN_EXCLUSIVE = 0, 1
+SORT_DESCENDING, SORT_FLOAT_TOTAL_ORDER = 1, 2
+VALUES_FROM_VIEW, VALUES_FROM_INDEX = 0, 1
+LOCATOR_IDENTITY, LOCATOR_MODULO = 0, 1
+
+EXPORTS = [
+    "ilgpu_hip_version", "ilgpu_hip_status_string",
+    "ilgpu_hip_last_runtime_error", "ilgpu_hip_radix_sort_temp_bytes",
+    "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
+    "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan",
+    "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
+]
+
+_NP_TO_TYPE = {
+    np.dtype(np.int8): I8, np.dtype(np.int16): I16, np.dtype(np.int32): I32,
+    np.dtype(np.int64): I64, np.dtype(np.uint8): U8, np.dtype(np.uint16): U16,
+    np.dtype(np.uint32): U32, np.dtype(np.uint64): U64,
+    np.dtype(np.float16): F16, np.dtype(np.float32): F32,
+    np.dtype(np.float64): F64,
+}
+
+
+def type_code(dtype) -> int:
+    return _NP_TO_TYPE[np.dtype(dtype)]
+
+
+# ---- errors: one class per .NET exception kind the C# layer would throw ----
+class HipAlgorithmsError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"{message} (status {status})")
+        self.status = status
+
+
+class ArgumentNullError(HipAlgorithmsError):
+    """ArgumentNullException: a view is null or empty."""
+
+
+class ArgumentOutOfRangeError(HipAlgorithmsError):
+    """ArgumentOutOfRangeException: output or temp too short, bad length."""
+
+
+class NotSupportedError(HipAlgorithmsError):
+    """NotSupportedException: 64-bit lengths, strides, unknown type or functor."""
+
+
+class InvalidOperationError(HipAlgorithmsError):
+    """InvalidOperationException: unaligned temp allocation."""
+
+
+class HipRuntimeError(HipAlgorithmsError):
+    """A HIP runtime call failed inside the library."""
+
+
+_ERRORS = {
+    ERROR_NULL_VIEW: ArgumentNullError,
+    ERROR_OUT_OF_RANGE: ArgumentOutOfRangeError,
+    ERROR_NOT_SUPPORTED: NotSupportedError,
+    ERROR_UNALIGNED_TEMP: InvalidOperationError,
+    ERROR_RUNTIME: HipRuntimeError,
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with "
+                "`python -m ilgpu_amd.build` (there is no fallback path)")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
+        p64 = ctypes.POINTER(ctypes.c_int64)
+        L.ilgpu_hip_version.restype = i32
+        L.ilgpu_hip_status_string.argtypes = [i32]
+        L.ilgpu_hip_status_string.restype = ctypes.c_char_p
+        L.ilgpu_hip_last_runtime_error.restype = i32
+        L.ilgpu_hip_radix_sort_temp_bytes.argtypes = [i64, i32, i32, p64]
+        L.ilgpu_hip_radix_sort_keys.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64]
+        L.ilgpu_hip_radix_sort_pairs.argtypes = [
+            vp, vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, i64]
+        L.ilgpu_hip_scan_temp_bytes.argtypes = [i64, i32, p64]
+        L.ilgpu_hip_scan.argtypes = [vp, vp, i64, i64, vp, i64, i64, i32, i32,
+                                     i32, vp, i64]
+        L.ilgpu_hip_reduce_temp_bytes.argtypes = [i64, i32, p64]
+        L.ilgpu_hip_reduce.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64, vp, i64]
+        L.ilgpu_hip_histogram.argtypes = [vp, vp, i64, i64, i32, vp, i64, i32,
+                                          i32, vp]
+        for name in EXPORTS:
+            if name.endswith(("_bytes", "_keys", "_pairs", "_scan", "_reduce",
+                              "_histogram")):
+                getattr(L, name).restype = i32
+        _lib = L
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return lib().ilgpu_hip_status_string(status).decode()
+
+
+def check(status: int) -> None:
+    if status != SUCCESS:
+        raise _ERRORS.get(status, HipAlgorithmsError)(status, status_string(status))
+
+
+# ---- device memory (torch as the allocator) --------------------------------
+class DeviceArray:
+    """``length`` elements of ``dtype`` in device memory."""
+
+    def __init__(self, length: int, dtype, *, _bytes=None):
+        import torch
+        self.dtype = np.dtype(dtype)
+        self.length = int(length)
+        nbytes = self.length * self.dtype.itemsize
+        self.bytes = _bytes if _bytes is not None else torch.empty(
+            max(nbytes, 1), dtype=torch.uint8, device="cuda:0")
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceArray":
+        import torch
+        a = np.ascontiguousarray(a)
+        host = torch.from_numpy(a.view(np.uint8).reshape(-1))
+        if host.numel() == 0:
+            return cls(0, a.dtype)
+        return cls(a.size, a.dtype, _bytes=host.to("cuda:0"))
+
+    @classmethod
+    def zeros(cls, length: int, dtype) -> "DeviceArray":
+        out = cls(length, dtype)
+        out.bytes.zero_()
+        return out
+
+    @property
+    def ptr(self) -> int:
+        return self.bytes.data_ptr() if self.length > 0 else 0
+
+    @property
+    def nbytes(self) -> int:
+        return self.length * self.dtype.itemsize
+
+    @property
+    def type_code(self) -> int:
+        return type_code(self.dtype)
+
+    def numpy(self) -> np.ndarray:
+        if self.length == 0:
+            return np.empty(0, dtype=self.dtype)
+        return self.bytes[: self.nbytes].cpu().numpy().view(self.dtype).copy()
+
+    def clone(self) -> "DeviceArray":
+        return DeviceArray(self.length, self.dtype, _bytes=self.bytes.clone())
+
+    def subview(self, offset: int, length: int) -> "DeviceArray":
+        """Elements [offset, offset+length) as a view on the same memory."""
+        s = self.dtype.itemsize
+        return DeviceArray(length, self.dtype,
+                           _bytes=self.bytes[offset * s:(offset + length) * s])
+
+
+def temp_buffer(nbytes: int) -> DeviceArray:
+    """An ``ArrayView<int>`` of at least ``nbytes`` bytes."""
+    return DeviceArray((nbytes + 3) // 4, np.int32)
+
+
+def _stream_ptr(stream) -> int:
+    if stream is None:
+        import torch
+        return torch.cuda.current_stream().cuda_stream
+    return getattr(stream, "cuda_stream", stream)
+
+
+def _query(fn, *args) -> int:
+    out = ctypes.c_int64(0)
+    check(fn(*args, ctypes.byref(out)))
+    return out.value
+
+
+# ---- thin wrappers, one per entry point -------------------------------------
+def radix_sort_temp_bytes(n: int, key_dtype, value_bytes: int = 0) -> int:
+    return _query(lib().ilgpu_hip_radix_sort_temp_bytes, n,
+                  type_code(key_dtype), value_bytes)
+
+
+def radix_sort_keys(keys: DeviceArray, temp: Optional[DeviceArray] = None, *,
+                    descending: bool = False, float_total_order: bool = False,
+                    stream=None, stride: int = 1) -> None:
+    if temp is None:
+        temp = temp_buffer(radix_sort_temp_bytes(keys.length, keys.dtype))
+    flags = (SORT_DESCENDING if descending else 0) | (
+        SORT_FLOAT_TOTAL_ORDER if float_total_order else 0)
+    check(lib().ilgpu_hip_radix_sort_keys(
+        _stream_ptr(stream), keys.ptr, keys.length, stride, keys.type_code,
+        flags, temp.ptr, temp.nbytes))
+
+
+def radix_sort_pairs(keys: DeviceArray, values: DeviceArray,
+                     temp: Optional[DeviceArray] = None, *,
+                     descending: bool = False, float_total_order: bool = False,
+                     values_from_index: bool = False, stream=None) -> None:
+    if temp is None:
+        temp = temp_buffer(radix_sort_temp_bytes(keys.length, keys.dtype,
+                                                 values.dtype.itemsize))
+    flags = (SORT_DESCENDING if descending else 0) | (
+        SORT_FLOAT_TOTAL_ORDER if float_total_order else 0)
+    if values.length != keys.length:
+        # RadixSortExtensions.cs:1053-1054
+        raise ArgumentOutOfRangeError(ERROR_OUT_OF_RANGE, "values")
+    check(lib().ilgpu_hip_radix_sort_pairs(
+        _stream_ptr(stream), keys.ptr, 1, values.ptr, 1, keys.length,
+        keys.type_code, values.dtype.itemsize, flags,
+        VALUES_FROM_INDEX if values_from_index else VALUES_FROM_VIEW,
+        temp.ptr, temp.nbytes))
+
+
+def scan_temp_bytes(n: int, dtype) -> int:
+    return _query(lib().ilgpu_hip_scan_temp_bytes, n, type_code(dtype))
+
+
+def scan(inp: DeviceArray, out: DeviceArray, temp: Optional[DeviceArray] = None,
+         *, op: int = OP_ADD, kind: int = SCAN_INCLUSIVE, stream=None) -> None:
+    if temp is None:
+        temp = temp_buffer(scan_temp_bytes(max(inp.length, 1), inp.dtype))
+    check(lib().ilgpu_hip_scan(
+        _stream_ptr(stream), inp.ptr, inp.length, 1, out.ptr, out.length, 1,
+        inp.type_code, op, kind, temp.ptr, temp.nbytes))
+
+
+def reduce_temp_bytes(n: int, dtype) -> int:
+    return _query(lib().ilgpu_hip_reduce_temp_bytes, n, type_code(dtype))
+
+
+def reduce(inp: DeviceArray, out: DeviceArray,
+           temp: Optional[DeviceArray] = None, *, op: int = OP_ADD,
+           stream=None) -> None:
+    if temp is None:
+        temp = temp_buffer(reduce_temp_bytes(max(inp.length, 1), inp.dtype))
+    check(lib().ilgpu_hip_reduce(
+        _stream_ptr(stream), inp.ptr, inp.length, 1, inp.type_code, op,
+        out.ptr, out.length, temp.ptr, temp.nbytes))
+
+
+def histogram(inp: DeviceArray, bins: DeviceArray,
+              overflow: Optional[DeviceArray] = None, *,
+              locator: int = LOCATOR_IDENTITY, stream=None) -> None:
+    check(lib().ilgpu_hip_histogram(
+        _stream_ptr(stream), inp.ptr, inp.length, 1, inp.type_code, bins.ptr,
+        bins.length, bins.type_code, locator,
+        overflow.ptr if overflow is not None else None))

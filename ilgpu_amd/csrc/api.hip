@@ -1,0 +1,242 @@
+// C ABI of libilgpu_hip_algorithms.so: argument validation (mirroring the
+// checks and exception kinds of the reference's host-side delegates) and
+// dispatch to the kernel launchers.  No GPU work is enqueued when validation
+// fails, and nothing here allocates device memory.
+#include <atomic>
+
+#include "kernels.hpp"
+
+namespace ilgpu_hip {
+
+namespace {
+thread_local int32_t g_last_runtime_error = 0;
+std::atomic<int> g_cu_count{0};
+}  // namespace
+
+void set_last_runtime_error(hipError_t e) { g_last_runtime_error = (int32_t)e; }
+
+int device_cu_count() {
+  int cached = g_cu_count.load(std::memory_order_relaxed);
+  if (cached > 0) return cached;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) !=
+          hipSuccess ||
+      cus <= 0)
+    cus = 256;
+  g_cu_count.store(cus, std::memory_order_relaxed);
+  return cus;
+}
+
+namespace {
+
+inline bool aligned_to(const void* p, int bytes) {
+  return (reinterpret_cast<uintptr_t>(p) % (uintptr_t)bytes) == 0;
+}
+
+// A view is valid when it has a buffer and a positive length
+// (ArrayView.IsValid, ArrayView.cs:261-265).
+inline bool valid_view(const void* p, int64_t length) {
+  return p != nullptr && length > 0;
+}
+
+// The checks TempViewManager makes on the caller's ArrayView<int> temp
+// (TempViewManager.cs:33-41, 84-89).
+inline int32_t check_temp(const void* temp, int64_t temp_bytes,
+                          int64_t required) {
+  if (temp == nullptr || temp_bytes <= 0) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!aligned_to(temp, 4)) return ILGPU_HIP_ERROR_UNALIGNED_TEMP;
+  if (temp_bytes < required) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  return ILGPU_HIP_SUCCESS;
+}
+
+inline bool scan_reduce_type(int32_t t) {
+  return t == ILGPU_HIP_I32 || t == ILGPU_HIP_I64 || t == ILGPU_HIP_U32 ||
+         t == ILGPU_HIP_U64 || t == ILGPU_HIP_F32 || t == ILGPU_HIP_F64;
+}
+
+inline bool valid_op(int32_t op) {
+  return op == ILGPU_HIP_OP_ADD || op == ILGPU_HIP_OP_MAX ||
+         op == ILGPU_HIP_OP_MIN;
+}
+
+}  // namespace
+}  // namespace ilgpu_hip
+
+using namespace ilgpu_hip;
+
+extern "C" {
+
+int32_t ilgpu_hip_version(void) { return ILGPU_HIP_ALGORITHMS_VERSION; }
+
+const char* ilgpu_hip_status_string(int32_t status) {
+  switch (status) {
+    case ILGPU_HIP_SUCCESS: return "success";
+    case ILGPU_HIP_ERROR_NULL_VIEW: return "invalid (null or empty) view";
+    case ILGPU_HIP_ERROR_OUT_OF_RANGE: return "argument out of range";
+    case ILGPU_HIP_ERROR_NOT_SUPPORTED: return "not supported";
+    case ILGPU_HIP_ERROR_UNALIGNED_TEMP: return "unaligned temp allocation";
+    case ILGPU_HIP_ERROR_RUNTIME: return "HIP runtime error";
+    default: return "unknown status";
+  }
+}
+
+int32_t ilgpu_hip_last_runtime_error(void) { return g_last_runtime_error; }
+
+/* ---- radix sort -------------------------------------------------------- */
+
+int32_t ilgpu_hip_radix_sort_temp_bytes(int64_t n, int32_t key_type,
+                                        int32_t value_bytes,
+                                        int64_t* temp_bytes) {
+  if (temp_bytes == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  const int kb = elem_size(key_type);
+  if (kb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (value_bytes != 0 && value_bytes != 1 && value_bytes != 2 &&
+      value_bytes != 4 && value_bytes != 8 && value_bytes != 16)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (n < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (n > radix_sort_max_length()) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  *temp_bytes = radix_sort_temp_bytes(n, kb, value_bytes);
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t ilgpu_hip_radix_sort_keys(ilgpu_hip_stream_t stream, void* keys,
+                                  int64_t n, int64_t stride, int32_t key_type,
+                                  int32_t flags, void* temp,
+                                  int64_t temp_bytes) {
+  const int kb = elem_size(key_type);
+  if (kb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(keys, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (n > radix_sort_max_length()) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (stride != 1 || !aligned_to(keys, kb)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (flags & ~(ILGPU_HIP_SORT_DESCENDING | ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int32_t rc = check_temp(temp, temp_bytes, radix_sort_temp_bytes(n, kb, 0));
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  SortArgs a{keys, nullptr, n, key_type, 0, flags, ILGPU_HIP_VALUES_FROM_VIEW, temp};
+  return launch_radix_sort(static_cast<hipStream_t>(stream), a);
+}
+
+int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void* keys,
+                                   int64_t key_stride, void* values,
+                                   int64_t value_stride, int64_t n,
+                                   int32_t key_type, int32_t value_bytes,
+                                   int32_t flags, int32_t value_source,
+                                   void* temp, int64_t temp_bytes) {
+  const int kb = elem_size(key_type);
+  if (kb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (value_bytes != 1 && value_bytes != 2 && value_bytes != 4 &&
+      value_bytes != 8 && value_bytes != 16)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(keys, n) || values == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (n > radix_sort_max_length()) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (key_stride != 1 || value_stride != 1 || !aligned_to(keys, kb) ||
+      !aligned_to(values, value_bytes))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (flags & ~(ILGPU_HIP_SORT_DESCENDING | ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (value_source != ILGPU_HIP_VALUES_FROM_VIEW &&
+      value_source != ILGPU_HIP_VALUES_FROM_INDEX)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (value_source == ILGPU_HIP_VALUES_FROM_INDEX && value_bytes != 4 &&
+      value_bytes != 8)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int32_t rc =
+      check_temp(temp, temp_bytes, radix_sort_temp_bytes(n, kb, value_bytes));
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  SortArgs a{keys, values, n, key_type, value_bytes, flags, value_source, temp};
+  return launch_radix_sort(static_cast<hipStream_t>(stream), a);
+}
+
+/* ---- scan -------------------------------------------------------------- */
+
+int32_t ilgpu_hip_scan_temp_bytes(int64_t n, int32_t elem_type,
+                                  int64_t* temp_bytes) {
+  if (temp_bytes == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!scan_reduce_type(elem_type)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (n < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (n > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  *temp_bytes = scan_temp_bytes(n, elem_size(elem_type));
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t ilgpu_hip_scan(ilgpu_hip_stream_t stream, const void* in,
+                       int64_t in_length, int64_t in_stride, void* out,
+                       int64_t out_length, int64_t out_stride,
+                       int32_t elem_type, int32_t op, int32_t kind, void* temp,
+                       int64_t temp_bytes) {
+  /* Order of checks as in ScanExtensions.cs:675-685. */
+  if (!scan_reduce_type(elem_type) || !valid_op(op) ||
+      (kind != ILGPU_HIP_SCAN_INCLUSIVE && kind != ILGPU_HIP_SCAN_EXCLUSIVE))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(in, in_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(out, out_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (out_length < in_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (in_length > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int eb = elem_size(elem_type);
+  if (in_stride != 1 || out_stride != 1 || !aligned_to(in, eb) ||
+      !aligned_to(out, eb))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int32_t rc = check_temp(temp, temp_bytes, scan_temp_bytes(in_length, eb));
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  return launch_scan(static_cast<hipStream_t>(stream), in, out, in_length,
+                     elem_type, op, kind, temp);
+}
+
+/* ---- reduce ------------------------------------------------------------ */
+
+int32_t ilgpu_hip_reduce_temp_bytes(int64_t n, int32_t elem_type,
+                                    int64_t* temp_bytes) {
+  if (temp_bytes == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!scan_reduce_type(elem_type)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (n < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  *temp_bytes = reduce_temp_bytes();
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t ilgpu_hip_reduce(ilgpu_hip_stream_t stream, const void* in, int64_t n,
+                         int64_t stride, int32_t elem_type, int32_t op,
+                         void* out, int64_t out_length, void* temp,
+                         int64_t temp_bytes) {
+  /* Order of checks as in ReductionExtensions.cs:146-153. */
+  if (!scan_reduce_type(elem_type) || !valid_op(op))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(in, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(out, out_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (n > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int eb = elem_size(elem_type);
+  if (stride != 1 || !aligned_to(in, eb) || !aligned_to(out, eb))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int32_t rc = check_temp(temp, temp_bytes, reduce_temp_bytes());
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  return launch_reduce(static_cast<hipStream_t>(stream), in, n, elem_type, op,
+                       out, temp);
+}
+
+/* ---- histogram --------------------------------------------------------- */
+
+int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void* in,
+                            int64_t n, int64_t stride, int32_t in_type,
+                            void* bins, int64_t num_bins, int32_t bin_type,
+                            int32_t locator, int32_t* overflow) {
+  /* Order of checks as in HistogramExtensions.cs:322-338. */
+  const int eb = elem_size(in_type);
+  if (eb < 0 || in_type == ILGPU_HIP_F16) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (bin_type != ILGPU_HIP_I32 && bin_type != ILGPU_HIP_U32 &&
+      bin_type != ILGPU_HIP_I64 && bin_type != ILGPU_HIP_U64)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (locator != ILGPU_HIP_LOCATOR_IDENTITY &&
+      locator != ILGPU_HIP_LOCATOR_MODULO)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(in, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(bins, num_bins)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (n > INT32_MAX || num_bins > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (stride != 1 || !aligned_to(in, eb) ||
+      !aligned_to(bins, elem_size(bin_type)) ||
+      (overflow != nullptr && !aligned_to(overflow, 4)))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  return launch_histogram(static_cast<hipStream_t>(stream), in, n, in_type,
+                          bins, num_bins, bin_type, locator, overflow);
+}
+
+}  // extern "C"

@@ -1,0 +1,44 @@
+// Internal launch interface between the C ABI (api.hip) and the kernel files.
+// All launchers assume validated arguments: non-null, naturally aligned
+// device pointers, 1 <= n <= INT32_MAX, stride 1, temp large enough.
+#pragma once
+
+#include "common.hpp"
+
+namespace ilgpu_hip {
+
+// reduce.hip
+int64_t reduce_temp_bytes();
+int32_t launch_reduce(hipStream_t stream, const void* in, int64_t n,
+                      int32_t type, int32_t op, void* out, void* temp);
+
+// scan.hip
+int64_t scan_temp_bytes(int64_t n, int elem_bytes);
+int32_t launch_scan(hipStream_t stream, const void* in, void* out, int64_t n,
+                    int32_t type, int32_t op, int32_t kind, void* temp);
+
+// histogram.hip
+int32_t launch_histogram(hipStream_t stream, const void* in, int64_t n,
+                         int32_t in_type, void* bins, int64_t num_bins,
+                         int32_t bin_type, int32_t locator, int32_t* overflow);
+
+// radix_sort.hip
+struct SortArgs {
+  void* keys;
+  void* values;      // nullptr for a keys-only sort
+  int64_t n;
+  int32_t key_type;
+  int32_t value_bytes;   // 0 for keys only
+  int32_t flags;
+  int32_t value_source;
+  void* temp;
+};
+int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes);
+int64_t radix_sort_max_length();
+int32_t launch_radix_sort(hipStream_t stream, const SortArgs& args);
+
+// fill kernel shared by scan and sort: words[0..count) = 0, as a kernel so
+// that callers may capture the stream into a graph.
+int32_t launch_zero_words(hipStream_t stream, uint32_t* words, int64_t count);
+
+}  // namespace ilgpu_hip

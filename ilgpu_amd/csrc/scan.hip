@@ -1,0 +1,363 @@
+// Inclusive / exclusive scan, single pass with decoupled look-back.
+//
+// Stands in for the Scan delegates of ScanExtensions.cs:930-959.  The
+// reference's single-pass kernel (ScanExtensions.cs:530-597) chains the groups
+// strictly through one global word (SequentialGroupExecutor.cs:58-77) and reads
+// the input twice; here each tile publishes its aggregate as soon as it has
+// it, and a tile's first wave resolves the prefix of up to 64 predecessor
+// tiles per step, so tiles only wait for data, never for their turn.
+//
+// Tile layout (kBlock = 256 threads, 4 waves, kVecs 16-byte vectors per lane):
+//   wave w owns a contiguous chunk of kVecs*64 vectors; vector j of lane l is
+//   chunk[j*64 + l], so every load/store instruction of a wave covers 1 KiB of
+//   consecutive addresses (dwordx4 per lane).  Scan order inside a wave is
+//   (j, lane, element): each lane scans its vector, the wave scans the vector
+//   totals once per j, and the running totals of earlier j are folded in.
+//
+// Tile ids come from a global ticket, so a tile's predecessors have always
+// started.  Status words are read and written with agent-scope atomics: the
+// eight XCDs of the device have separate L2s.
+//   4-byte T: one 64-bit word {flag, value} per tile;
+//   8-byte T: a flag word (release/acquire) and two value slots per tile.
+//
+// Algorithmic HBM traffic: 2 * n * sizeof(T) bytes (status words: 8 B/tile).
+#include "kernels.hpp"
+
+namespace ilgpu_hip {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWaveSize;
+constexpr int kVecs = 4;
+constexpr uint32_t kFlagInvalid = 0, kFlagAggregate = 1, kFlagPrefix = 2;
+constexpr int64_t kHeaderBytes = 256;  // ticket counter, padded
+
+template <typename T> constexpr int tile_elems() {
+  return kBlock * kVecs * Vec16<T>::N;
+}
+
+template <typename T> struct Bits;
+template <> struct Bits<int32_t> { using type = uint32_t; };
+template <> struct Bits<uint32_t> { using type = uint32_t; };
+template <> struct Bits<float> { using type = uint32_t; };
+template <> struct Bits<int64_t> { using type = uint64_t; };
+template <> struct Bits<uint64_t> { using type = uint64_t; };
+template <> struct Bits<double> { using type = uint64_t; };
+
+template <typename T>
+__device__ __forceinline__ typename Bits<T>::type to_bits(T v) {
+  typename Bits<T>::type b;
+  __builtin_memcpy(&b, &v, sizeof(T));
+  return b;
+}
+template <typename T>
+__device__ __forceinline__ T from_bits(typename Bits<T>::type b) {
+  T v;
+  __builtin_memcpy(&v, &b, sizeof(T));
+  return v;
+}
+
+// Look-back state in temp memory.
+template <typename T, int SIZE = sizeof(T)> struct TileState;
+
+template <typename T> struct TileState<T, 4> {
+  uint64_t* words;
+  __device__ __forceinline__ void publish(int tile, uint32_t flag, T v) const {
+    const uint64_t w = ((uint64_t)flag << 32) | to_bits(v);
+    __hip_atomic_store(&words[tile], w, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // Spins until the tile has published something; returns its flag.
+  __device__ __forceinline__ uint32_t wait(int tile, T* v) const {
+    uint64_t w;
+    while (true) {
+      w = __hip_atomic_load(&words[tile], __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+      if ((uint32_t)(w >> 32) != kFlagInvalid) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    *v = from_bits<T>((uint32_t)w);
+    return (uint32_t)(w >> 32);
+  }
+};
+
+template <typename T> struct TileState<T, 8> {
+  uint32_t* flags;
+  uint64_t* aggregates;
+  uint64_t* prefixes;
+  __device__ __forceinline__ void publish(int tile, uint32_t flag, T v) const {
+    uint64_t* slot = flag == kFlagPrefix ? prefixes : aggregates;
+    __hip_atomic_store(&slot[tile], to_bits(v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&flags[tile], flag, __ATOMIC_RELEASE,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __device__ __forceinline__ uint32_t wait(int tile, T* v) const {
+    uint32_t f;
+    while (true) {
+      f = __hip_atomic_load(&flags[tile], __ATOMIC_ACQUIRE,
+                            __HIP_MEMORY_SCOPE_AGENT);
+      if (f != kFlagInvalid) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    const uint64_t* slot = f == kFlagPrefix ? prefixes : aggregates;
+    *v = from_bits<T>(__hip_atomic_load(&slot[tile], __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT));
+    return f;
+  }
+};
+
+template <typename T, int OP>
+__device__ __forceinline__ T wave_inclusive_scan(T v, int lane) {
+  using F = Functor<T, OP>;
+#pragma unroll
+  for (int d = 1; d < kWaveSize; d <<= 1) {
+    T o = shfl_up(v, d);
+    if (lane >= d) v = F::apply(o, v);
+  }
+  return v;
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ T wave_reduce(T v) {
+  using F = Functor<T, OP>;
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1)
+    v = F::apply(v, shfl_down(v, off));
+  return shfl(v, 0);
+}
+
+// Executed by the first wave of the block.  Publishes the tile's aggregate,
+// resolves the exclusive prefix of the tile and publishes the inclusive one.
+template <typename T, int OP>
+__device__ __forceinline__ T resolve_prefix(const TileState<T>& st, int tile,
+                                            T aggregate, int lane) {
+  using F = Functor<T, OP>;
+  if (tile == 0) {
+    if (lane == 0) st.publish(0, kFlagPrefix, aggregate);
+    return F::identity();
+  }
+  if (lane == 0) st.publish(tile, kFlagAggregate, aggregate);
+  T exclusive = F::identity();
+  int base = tile - 1;
+  while (true) {
+    const int idx = base - lane;
+    T val = F::identity();
+    uint32_t flag = kFlagPrefix;  // virtual prefix in front of tile 0
+    if (idx >= 0) flag = st.wait(idx, &val);
+    const uint64_t has_prefix = __ballot(flag == kFlagPrefix);
+    // Lanes run from the nearest predecessor (lane 0) to the farthest; the
+    // first lane holding an inclusive prefix ends the walk.
+    const int first = has_prefix != 0
+                          ? __ffsll((unsigned long long)has_prefix) - 1
+                          : kWaveSize - 1;
+    const T contrib = lane <= first ? val : F::identity();
+    exclusive = F::apply(wave_reduce<T, OP>(contrib), exclusive);
+    if (has_prefix != 0) break;  // wave-uniform
+    base -= kWaveSize;
+  }
+  if (lane == 0) st.publish(tile, kFlagPrefix, F::apply(exclusive, aggregate));
+  return exclusive;
+}
+
+template <typename T, int OP, bool VECTOR>
+__global__ __launch_bounds__(kBlock) void scan_kernel(
+    const T* __restrict__ in, T* __restrict__ out, int64_t n, int inclusive,
+    uint32_t* __restrict__ ticket, TileState<T> st) {
+  using F = Functor<T, OP>;
+  using V = typename Vec16<T>::type;
+  constexpr int VN = Vec16<T>::N;
+  constexpr int kTile = tile_elems<T>();
+  constexpr int kWaveElems = kTile / kWaves;
+
+  __shared__ int s_tile;
+  __shared__ T s_wave_total[kWaves];
+  __shared__ T s_prefix;
+
+  if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
+  __syncthreads();
+  const int tile = s_tile;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  const int64_t tile_base = (int64_t)tile * kTile;
+  const int64_t wave_base = tile_base + (int64_t)wave * kWaveElems;
+  const bool full = tile_base + kTile <= n;
+
+  T x[kVecs][VN];
+  if (VECTOR && full) {
+    const V* src = reinterpret_cast<const V*>(in + wave_base);
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j) {
+      V v = __builtin_nontemporal_load(&src[j * kWaveSize + lane]);
+#pragma unroll
+      for (int k = 0; k < VN; ++k) x[j][k] = v[k];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j)
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
+        x[j][k] = idx < n ? in[idx] : F::identity();
+      }
+  }
+
+  // Lane-local inclusive scan of each vector, then one wave scan per j.
+  T lane_excl[kVecs];   // fold of the vectors of lower lanes, same j
+  T seg_total[kVecs];   // fold of the whole 64-lane row j
+#pragma unroll
+  for (int j = 0; j < kVecs; ++j) {
+#pragma unroll
+    for (int k = 1; k < VN; ++k) x[j][k] = F::apply(x[j][k - 1], x[j][k]);
+    const T inc = wave_inclusive_scan<T, OP>(x[j][VN - 1], lane);
+    seg_total[j] = shfl(inc, kWaveSize - 1);
+    const T up = shfl_up(inc, 1);
+    lane_excl[j] = lane == 0 ? F::identity() : up;
+  }
+  T wave_total = seg_total[0];
+#pragma unroll
+  for (int j = 1; j < kVecs; ++j) wave_total = F::apply(wave_total, seg_total[j]);
+  if (lane == 0) s_wave_total[wave] = wave_total;
+  __syncthreads();
+
+  T wave_prefix = F::identity();
+  T block_total = s_wave_total[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) {
+    if (w == wave) wave_prefix = block_total;
+    block_total = F::apply(block_total, s_wave_total[w]);
+  }
+
+  if (wave == 0) {
+    const T exclusive = resolve_prefix<T, OP>(st, tile, block_total, lane);
+    if (lane == 0) s_prefix = exclusive;
+  }
+  __syncthreads();
+
+  T running = F::apply(s_prefix, wave_prefix);  // prefix of row 0 of this wave
+  V* dst = reinterpret_cast<V*>(out + wave_base);
+#pragma unroll
+  for (int j = 0; j < kVecs; ++j) {
+    const T before = F::apply(running, lane_excl[j]);  // prefix of x[j][0]
+    T r[VN];
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      if (inclusive) r[k] = F::apply(before, x[j][k]);
+      else r[k] = k == 0 ? before : F::apply(before, x[j][k - 1]);
+    }
+    if (VECTOR && full) {
+      V v;
+#pragma unroll
+      for (int k = 0; k < VN; ++k) v[k] = r[k];
+      dst[j * kWaveSize + lane] = v;
+    } else {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
+        if (idx < n) out[idx] = r[k];
+      }
+    }
+    running = F::apply(running, seg_total[j]);
+  }
+}
+
+__global__ void zero_words_kernel(uint32_t* words, int64_t count) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count;
+       i += stride)
+    words[i] = 0u;
+}
+
+template <typename T> int64_t num_tiles(int64_t n) {
+  return div_up(n, tile_elems<T>());
+}
+
+template <typename T, int OP>
+int32_t launch_typed(hipStream_t stream, const void* in, void* out, int64_t n,
+                     int32_t kind, void* temp) {
+  const int64_t tiles = num_tiles<T>(n);
+  char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)temp, 256));
+  uint32_t* ticket = reinterpret_cast<uint32_t*>(base);
+  TileState<T> st;
+  int64_t zero_words;
+  if constexpr (sizeof(T) == 4) {
+    st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
+    zero_words = (kHeaderBytes + tiles * 8) / 4;
+  } else {
+    const int64_t flag_bytes = align_up(tiles * 4, 256);
+    st.flags = reinterpret_cast<uint32_t*>(base + kHeaderBytes);
+    st.aggregates = reinterpret_cast<uint64_t*>(base + kHeaderBytes + flag_bytes);
+    st.prefixes = st.aggregates + tiles;
+    zero_words = (kHeaderBytes + flag_bytes) / 4;
+  }
+  int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
+                                 zero_words);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  const bool vector = (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  const int inclusive = kind == ILGPU_HIP_SCAN_INCLUSIVE ? 1 : 0;
+  if (vector) {
+    hipLaunchKernelGGL((scan_kernel<T, OP, true>), dim3((unsigned)tiles),
+                       dim3(kBlock), 0, stream, static_cast<const T*>(in),
+                       static_cast<T*>(out), n, inclusive, ticket, st);
+  } else {
+    hipLaunchKernelGGL((scan_kernel<T, OP, false>), dim3((unsigned)tiles),
+                       dim3(kBlock), 0, stream, static_cast<const T*>(in),
+                       static_cast<T*>(out), n, inclusive, ticket, st);
+  }
+  ILGPU_HIP_CHECK(hipGetLastError());
+  return ILGPU_HIP_SUCCESS;
+}
+
+template <typename T>
+int32_t launch_op(hipStream_t stream, const void* in, void* out, int64_t n,
+                  int32_t op, int32_t kind, void* temp) {
+  switch (op) {
+    case ILGPU_HIP_OP_ADD:
+      return launch_typed<T, ILGPU_HIP_OP_ADD>(stream, in, out, n, kind, temp);
+    case ILGPU_HIP_OP_MAX:
+      return launch_typed<T, ILGPU_HIP_OP_MAX>(stream, in, out, n, kind, temp);
+    case ILGPU_HIP_OP_MIN:
+      return launch_typed<T, ILGPU_HIP_OP_MIN>(stream, in, out, n, kind, temp);
+    default:
+      return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  }
+}
+
+}  // namespace
+
+int32_t launch_zero_words(hipStream_t stream, uint32_t* words, int64_t count) {
+  if (count <= 0) return ILGPU_HIP_SUCCESS;
+  int64_t blocks = div_up(count, 256 * 4);
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     stream, words, count);
+  ILGPU_HIP_CHECK(hipGetLastError());
+  return ILGPU_HIP_SUCCESS;
+}
+
+int64_t scan_temp_bytes(int64_t n, int elem_bytes) {
+  // 256 bytes of alignment slack + header + per-tile state.
+  if (elem_bytes == 4) {
+    const int64_t tiles = num_tiles<uint32_t>(n);
+    return 256 + kHeaderBytes + tiles * 8;
+  }
+  const int64_t tiles = num_tiles<uint64_t>(n);
+  return 256 + kHeaderBytes + align_up(tiles * 4, 256) + tiles * 16;
+}
+
+int32_t launch_scan(hipStream_t stream, const void* in, void* out, int64_t n,
+                    int32_t type, int32_t op, int32_t kind, void* temp) {
+  switch (type) {
+    case ILGPU_HIP_I32: return launch_op<int32_t>(stream, in, out, n, op, kind, temp);
+    case ILGPU_HIP_U32: return launch_op<uint32_t>(stream, in, out, n, op, kind, temp);
+    case ILGPU_HIP_I64: return launch_op<int64_t>(stream, in, out, n, op, kind, temp);
+    case ILGPU_HIP_U64: return launch_op<uint64_t>(stream, in, out, n, op, kind, temp);
+    case ILGPU_HIP_F32: return launch_op<float>(stream, in, out, n, op, kind, temp);
+    case ILGPU_HIP_F64: return launch_op<double>(stream, in, out, n, op, kind, temp);
+    default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  }
+}
+
+}  // namespace ilgpu_hip

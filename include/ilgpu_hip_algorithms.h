@@ -1,0 +1,191 @@
+/*
+ * ilgpu_hip_algorithms.h — C ABI of libilgpu_hip_algorithms.so
+ *
+ * Hand-written gfx950 (MI355X, CDNA4) implementation of the data-parallel
+ * primitives of ILGPU.Algorithms: radix sort (keys, key/value pairs), inclusive
+ * and exclusive scan, reduction and histogram.  The entry points below are
+ * what a P/Invoke layer behind ILGPU's existing C# surface binds; each one
+ * names the reference interface it stands in for (paths relative to the ILGPU
+ * source tree).
+ *
+ * Conventions
+ *  - Every pointer named keys/values/in/out/bins/overflow/temp is a DEVICE
+ *    pointer to memory the caller owns (the address an ArrayView yields from
+ *    LoadEffectiveAddressAsPtr, ArrayViewExtensions.cs:48-50).
+ *  - `stream` is a hipStream_t (NULL = the default stream).  All work is
+ *    enqueued asynchronously on it, like the reference's delegates; the
+ *    caller synchronises before reading results.
+ *  - Lengths and strides count ELEMENTS.  Only stride == 1 (Stride1D.Dense,
+ *    or Stride1D.General with stride 1 as the reference's tests use) is
+ *    accepted; anything else returns ILGPU_HIP_ERROR_NOT_SUPPORTED.
+ *  - Lengths above INT32_MAX return ILGPU_HIP_ERROR_NOT_SUPPORTED, like
+ *    ErrorMessages.NotSupportedArrayView64 in the reference.
+ *  - The library allocates no device memory and keeps no pointer after a call
+ *    returns.  Scratch space comes from `temp` (the reference's
+ *    ArrayView<int> temp), sized by the *_temp_bytes queries; its contents on
+ *    entry are irrelevant and on exit undefined.  One in-flight call per temp
+ *    buffer; calls on different streams with different temps may overlap.
+ *  - Return value: ilgpu_hip_status (0 = success).  Argument errors are
+ *    detected before any GPU work is enqueued.
+ */
+#ifndef ILGPU_HIP_ALGORITHMS_H
+#define ILGPU_HIP_ALGORITHMS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ILGPU_HIP_ALGORITHMS_VERSION 100 /* major*10000 + minor*100 + patch */
+
+typedef void *ilgpu_hip_stream_t; /* hipStream_t */
+
+/* Status codes and the .NET exception each maps to in the C# layer. */
+typedef enum ilgpu_hip_status {
+  ILGPU_HIP_SUCCESS = 0,
+  ILGPU_HIP_ERROR_NULL_VIEW = 1,      /* ArgumentNullException: invalid view */
+  ILGPU_HIP_ERROR_OUT_OF_RANGE = 2,   /* ArgumentOutOfRangeException */
+  ILGPU_HIP_ERROR_NOT_SUPPORTED = 3,  /* NotSupportedException */
+  ILGPU_HIP_ERROR_UNALIGNED_TEMP = 4, /* InvalidOperationException
+                                         (TempViewManager.cs:98-106) */
+  ILGPU_HIP_ERROR_RUNTIME = 5         /* a HIP call failed; see
+                                         ilgpu_hip_last_runtime_error() */
+} ilgpu_hip_status;
+
+/* Element types: NumericTypes of TypeInformation.ttinclude:94-121. */
+typedef enum ilgpu_hip_type {
+  ILGPU_HIP_I8 = 0, ILGPU_HIP_I16 = 1, ILGPU_HIP_I32 = 2, ILGPU_HIP_I64 = 3,
+  ILGPU_HIP_U8 = 4, ILGPU_HIP_U16 = 5, ILGPU_HIP_U32 = 6, ILGPU_HIP_U64 = 7,
+  ILGPU_HIP_F16 = 8, ILGPU_HIP_F32 = 9, ILGPU_HIP_F64 = 10
+} ilgpu_hip_type;
+
+/* Scan/reduce functors: Add/Max/Min of ScanReduceOperations.tt:20-27. */
+typedef enum ilgpu_hip_op {
+  ILGPU_HIP_OP_ADD = 0, ILGPU_HIP_OP_MAX = 1, ILGPU_HIP_OP_MIN = 2
+} ilgpu_hip_op;
+
+/* ScanKind (ScanExtensions.cs:27-38). */
+typedef enum ilgpu_hip_scan_kind {
+  ILGPU_HIP_SCAN_INCLUSIVE = 0, ILGPU_HIP_SCAN_EXCLUSIVE = 1
+} ilgpu_hip_scan_kind;
+
+/* Sort flags.  DESCENDING selects the Descending* functor
+ * (RadixSortOperations.tt:98-125).  By default floating-point keys are
+ * ordered exactly as the reference's ExtractRadixBits orders them
+ * (RadixSortOperations.tt:81-89, including what it does to negative values);
+ * FLOAT_TOTAL_ORDER instead sorts them in IEEE-754 totalOrder and has no
+ * counterpart in the reference. */
+enum {
+  ILGPU_HIP_SORT_DESCENDING = 1,
+  ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER = 2
+};
+
+/* Where the values of a key/value sort come from: the values view itself
+ * (ViewSourceSequencer, Sequencer.cs:79-102) or value[i] = (TValue)i computed
+ * on the fly (IndexSequencer / Int32Sequencer ... , Sequencer.cs:36-45,
+ * Sequencers.tt:25-37; integer value types of 4 or 8 bytes). */
+typedef enum ilgpu_hip_value_source {
+  ILGPU_HIP_VALUES_FROM_VIEW = 0,
+  ILGPU_HIP_VALUES_FROM_INDEX = 1
+} ilgpu_hip_value_source;
+
+/* Histogram bin locators (IComputeSingleBinOperation, IHistogramOperations.cs:
+ * 19-30, is arbitrary user code in the reference; a native library offers a
+ * closed set).  IDENTITY: bin = (int)value, elements outside [0, num_bins)
+ * are ignored.  MODULO: bin = |value % num_bins|, the locator of the
+ * reference's own tests (HistogramTests.tt:83-94). */
+typedef enum ilgpu_hip_locator {
+  ILGPU_HIP_LOCATOR_IDENTITY = 0,
+  ILGPU_HIP_LOCATOR_MODULO = 1
+} ilgpu_hip_locator;
+
+/* ---- library ----------------------------------------------------------- */
+
+int32_t ilgpu_hip_version(void);
+const char *ilgpu_hip_status_string(int32_t status);
+/* hipError_t of the most recent failing HIP call on the calling thread. */
+int32_t ilgpu_hip_last_runtime_error(void);
+
+/* ---- radix sort ---------------------------------------------------------
+ * Replaces: RadixSort<T,TStride> delegates made by CreateRadixSort
+ * (RadixSortExtensions.cs:37-42, 1130-1337), RadixSortPairs delegates made by
+ * CreateRadixSortPairs (:56-96, 1017-1118) and the sizing helpers
+ * ComputeRadixSortTempStorageSize / ComputeRadixSortPairsTempStorageSize
+ * (:384-447).  Sorting is in place and stable; a pairs sort permutes `values`
+ * with the keys.
+ */
+
+/* Bytes of temp needed to sort n keys of key_type, each with a payload of
+ * value_bytes bytes (0 for a keys-only sort).  64-bit arithmetic throughout
+ * (the reference's pair sizing multiplies in 32 bits). */
+int32_t ilgpu_hip_radix_sort_temp_bytes(int64_t n, int32_t key_type,
+                                        int32_t value_bytes,
+                                        int64_t *temp_bytes);
+
+int32_t ilgpu_hip_radix_sort_keys(ilgpu_hip_stream_t stream, void *keys,
+                                  int64_t n, int64_t stride, int32_t key_type,
+                                  int32_t flags, void *temp,
+                                  int64_t temp_bytes);
+
+/* value_bytes in {1, 2, 4, 8, 16}.  With ILGPU_HIP_VALUES_FROM_INDEX the
+ * incoming contents of `values` are ignored and value_bytes must be 4 or 8. */
+int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void *keys,
+                                   int64_t key_stride, void *values,
+                                   int64_t value_stride, int64_t n,
+                                   int32_t key_type, int32_t value_bytes,
+                                   int32_t flags, int32_t value_source,
+                                   void *temp, int64_t temp_bytes);
+
+/* ---- scan ---------------------------------------------------------------
+ * Replaces: Scan<T,TStrideIn,TStrideOut> delegates made by CreateScan(kind)
+ * (ScanExtensions.cs:52-61, 930-959) and ComputeScanTempStorageSize (:158-170).
+ * elem_type in {I32, I64, U32, U64, F32, F64}.  out_length may exceed
+ * in_length (only the first in_length outputs are written, :679-680);
+ * shorter is ILGPU_HIP_ERROR_OUT_OF_RANGE.  in and out must not overlap
+ * unless they are identical.
+ */
+int32_t ilgpu_hip_scan_temp_bytes(int64_t n, int32_t elem_type,
+                                  int64_t *temp_bytes);
+
+int32_t ilgpu_hip_scan(ilgpu_hip_stream_t stream, const void *in,
+                       int64_t in_length, int64_t in_stride, void *out,
+                       int64_t out_length, int64_t out_stride,
+                       int32_t elem_type, int32_t op, int32_t kind, void *temp,
+                       int64_t temp_bytes);
+
+/* ---- reduce -------------------------------------------------------------
+ * Replaces: Reduction<T,TStride> delegates made by CreateReduction and the
+ * Reduce overloads (ReductionExtensions.cs:30-35, 135-216).  out[0] is
+ * overwritten with the fold of all inputs (:158-159); out_length >= 1.
+ * Integer results are exact (wrapping adds); floating-point Add accumulates
+ * in float64 in a fixed order, so repeated calls give identical bits.
+ * The reference's delegate has no temp argument: the P/Invoke layer owns a
+ * small scratch buffer of ilgpu_hip_reduce_temp_bytes() per delegate.
+ */
+int32_t ilgpu_hip_reduce_temp_bytes(int64_t n, int32_t elem_type,
+                                    int64_t *temp_bytes);
+
+int32_t ilgpu_hip_reduce(ilgpu_hip_stream_t stream, const void *in,
+                         int64_t n, int64_t stride, int32_t elem_type,
+                         int32_t op, void *out, int64_t out_length, void *temp,
+                         int64_t temp_bytes);
+
+/* ---- histogram ----------------------------------------------------------
+ * Replaces: Histogram / HistogramUnchecked delegates and launchers
+ * (HistogramExtensions.cs:35-59, 293-508; HistogramLaunchers.tt:52-101).
+ * bins[locator(v)] += 1 for every input element; bins are ACCUMULATED into,
+ * never cleared.  bin_type in {I32, I64, U32, U64}.  If `overflow` is not
+ * NULL, overflow[0] |= 1 when some bin's count passed the bin type's MaxValue
+ * (HistogramOperations.tt:36-40); NULL selects the unchecked variant.
+ * in_type: any ilgpu_hip_type except F16.
+ */
+int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void *in,
+                            int64_t n, int64_t stride, int32_t in_type,
+                            void *bins, int64_t num_bins, int32_t bin_type,
+                            int32_t locator, int32_t *overflow);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ILGPU_HIP_ALGORITHMS_H */

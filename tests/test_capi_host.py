@@ -1,0 +1,158 @@
+"""Host-only checks of the C ABI: the library loads, exports every symbol the
+header declares, sizes temp storage sensibly and rejects bad arguments with
+the documented status before touching the GPU.  No compute calls."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from ilgpu_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ilgpu_hip_algorithms.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ilgpu_hip_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = capi.lib()
+    names = declared_functions()
+    assert len(names) >= 11
+    for name in names:
+        assert hasattr(L, name), name
+    assert sorted(capi.EXPORTS) == names
+
+
+def test_version_and_status_strings():
+    assert capi.lib().ilgpu_hip_version() == 100
+    for status in range(6):
+        assert capi.status_string(status) != "unknown status"
+    assert capi.status_string(99) == "unknown status"
+
+
+def test_temp_size_queries():
+    n = 1 << 20
+    keys_only = capi.radix_sort_temp_bytes(n, np.uint32)
+    assert keys_only >= n * 4
+    with_values = capi.radix_sort_temp_bytes(n, np.uint32, 4)
+    assert with_values >= keys_only + n * 4
+    # 2^27 pairs of (u64, u32): the size the reference's own helper overflows
+    # on (RadixSortExtensions.cs:400-402) is computed in 64 bits here.
+    big = capi.radix_sort_temp_bytes(1 << 27, np.uint64, 4)
+    assert big > (1 << 27) * 12
+    assert capi.scan_temp_bytes(n, np.int32) < n  # a few bytes per tile
+    assert capi.scan_temp_bytes(n, np.float64) < n
+    assert capi.reduce_temp_bytes(n, np.float32) <= 64 * 1024
+    assert capi.reduce_temp_bytes(1, np.float32) == capi.reduce_temp_bytes(n, np.float32)
+
+
+def test_temp_size_query_errors():
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.radix_sort_temp_bytes(0, np.uint32)
+    with pytest.raises(capi.NotSupportedError):
+        capi.radix_sort_temp_bytes(16, np.uint32, 3)
+    with pytest.raises(capi.NotSupportedError):
+        capi.scan_temp_bytes(16, np.int16)  # not a scan/reduce type
+    with pytest.raises(capi.NotSupportedError):
+        capi.scan_temp_bytes(1 << 31, np.int32)  # NotSupportedArrayView64
+    out = ctypes.c_int64()
+    assert capi.lib().ilgpu_hip_radix_sort_temp_bytes(
+        16, 99, 0, ctypes.byref(out)) == capi.ERROR_NOT_SUPPORTED
+
+
+FAKE = 0x10000  # a non-null, 16-byte aligned "device pointer" that is never dereferenced
+
+
+def test_sort_argument_validation():
+    L = capi.lib()
+    big = 1 << 40
+    # invalid (null / empty) views -> ArgumentNullException
+    assert L.ilgpu_hip_radix_sort_keys(None, None, 16, 1, capi.U32, 0, FAKE, big) == capi.ERROR_NULL_VIEW
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 0, 1, capi.U32, 0, FAKE, big) == capi.ERROR_NULL_VIEW
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 0, None, big) == capi.ERROR_NULL_VIEW
+    # temp too small -> ArgumentOutOfRangeException (TempViewManager.cs:88-89)
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 0, FAKE, 8) == capi.ERROR_OUT_OF_RANGE
+    # temp not int-aligned -> InvalidOperationException
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 0, FAKE + 2, big) == capi.ERROR_UNALIGNED_TEMP
+    # 64-bit lengths, strides, unknown types/flags -> NotSupportedException
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 1 << 31, 1, capi.U32, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 2, capi.U32, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, 42, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 8, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    # pairs
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, None, 1, 16, capi.U32, 4, 0, 0, FAKE, big) == capi.ERROR_NULL_VIEW
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 3, 0, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 2, 0, capi.VALUES_FROM_INDEX, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 4, 0, 0, FAKE, 64) == capi.ERROR_OUT_OF_RANGE
+
+
+def test_scan_argument_validation():
+    L = capi.lib()
+    big = 1 << 40
+    args = dict(t=capi.I32, op=capi.OP_ADD, kind=capi.SCAN_INCLUSIVE)
+
+    def call(inp=FAKE, n_in=16, s_in=1, out=FAKE, n_out=16, s_out=1, t=args["t"],
+             op=args["op"], kind=args["kind"], temp=FAKE, tb=big):
+        return L.ilgpu_hip_scan(None, inp, n_in, s_in, out, n_out, s_out, t, op,
+                                kind, temp, tb)
+
+    assert call(inp=None) == capi.ERROR_NULL_VIEW
+    assert call(out=None) == capi.ERROR_NULL_VIEW
+    assert call(n_in=0) == capi.ERROR_NULL_VIEW
+    assert call(n_out=8) == capi.ERROR_OUT_OF_RANGE        # ScanExtensions.cs:679-680
+    assert call(n_in=1 << 31, n_out=1 << 31) == capi.ERROR_NOT_SUPPORTED
+    assert call(s_in=2) == capi.ERROR_NOT_SUPPORTED
+    assert call(t=capi.U8) == capi.ERROR_NOT_SUPPORTED
+    assert call(op=7) == capi.ERROR_NOT_SUPPORTED
+    assert call(kind=5) == capi.ERROR_NOT_SUPPORTED
+    assert call(temp=None) == capi.ERROR_NULL_VIEW
+    assert call(tb=4) == capi.ERROR_OUT_OF_RANGE
+
+
+def test_reduce_argument_validation():
+    L = capi.lib()
+    big = 1 << 20
+
+    def call(inp=FAKE, n=16, stride=1, t=capi.F32, op=capi.OP_ADD, out=FAKE,
+             n_out=1, temp=FAKE, tb=big):
+        return L.ilgpu_hip_reduce(None, inp, n, stride, t, op, out, n_out, temp, tb)
+
+    assert call(inp=None) == capi.ERROR_NULL_VIEW
+    assert call(n=0) == capi.ERROR_NULL_VIEW
+    assert call(out=None) == capi.ERROR_NULL_VIEW
+    assert call(n_out=0) == capi.ERROR_NULL_VIEW
+    assert call(n=1 << 31) == capi.ERROR_NOT_SUPPORTED
+    assert call(t=capi.I16) == capi.ERROR_NOT_SUPPORTED
+    assert call(stride=3) == capi.ERROR_NOT_SUPPORTED
+    assert call(tb=16) == capi.ERROR_OUT_OF_RANGE
+
+
+def test_histogram_argument_validation():
+    L = capi.lib()
+
+    def call(inp=FAKE, n=16, stride=1, t=capi.U8, bins=FAKE, nb=256,
+             bt=capi.I32, loc=capi.LOCATOR_IDENTITY, ov=FAKE):
+        return L.ilgpu_hip_histogram(None, inp, n, stride, t, bins, nb, bt, loc, ov)
+
+    assert call(inp=None) == capi.ERROR_NULL_VIEW
+    assert call(n=0) == capi.ERROR_NULL_VIEW
+    assert call(bins=None) == capi.ERROR_NULL_VIEW
+    assert call(nb=0) == capi.ERROR_NULL_VIEW
+    assert call(n=1 << 31) == capi.ERROR_NOT_SUPPORTED
+    assert call(t=capi.F16) == capi.ERROR_NOT_SUPPORTED
+    assert call(bt=capi.F32) == capi.ERROR_NOT_SUPPORTED
+    assert call(loc=9) == capi.ERROR_NOT_SUPPORTED
+    assert call(stride=2) == capi.ERROR_NOT_SUPPORTED
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", "/nonexistent/libilgpu_hip_algorithms.so")
+    with pytest.raises(FileNotFoundError):
+        capi.lib()

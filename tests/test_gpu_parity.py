@@ -1,0 +1,464 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU
+oracle on the same inputs.  Bit-exact for every integer result (sort, scan,
+reduce, histogram) and for stable pair order; floating-point sums within the
+tolerance written in each test."""
+import sys
+
+import numpy as np
+import pytest
+
+from ilgpu_amd import capi, datagen
+from oracle import cpu_oracle as O
+from tests.refcases import (ALL_KEY_DTYPES, ARRAY_SIZES, ATOMIC_NUMERIC_DTYPES,
+                            compute_inverted_sequence, compute_sequence)
+
+pytestmark = pytest.mark.gpu
+
+D = capi.DeviceArray
+INT_KEY_DTYPES = [d for d in ALL_KEY_DTYPES if np.dtype(d).kind in "iu"]
+SCAN_DTYPES = ATOMIC_NUMERIC_DTYPES
+OPS = [capi.OP_ADD, capi.OP_MAX, capi.OP_MIN]
+
+
+def note(*args):
+    print(*args, flush=True)
+    sys.stdout.flush()
+
+
+def sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def random_ints(dtype, n, seed=0, lo=None, hi=None):
+    info = np.iinfo(dtype)
+    lo = info.min if lo is None else lo
+    hi = info.max if hi is None else hi
+    return np.random.default_rng(seed).integers(lo, hi, size=n, dtype=dtype,
+                                                endpoint=True)
+
+
+def random_float_bits(dtype, n, seed=0):
+    """Arbitrary bit patterns (includes negatives, NaNs, infinities, -0)."""
+    u = {2: np.uint16, 4: np.uint32, 8: np.uint64}[np.dtype(dtype).itemsize]
+    return random_ints(u, n, seed).view(dtype)
+
+
+# ------------------------------------------------------------------- reduce
+def gpu_reduce(values, op):
+    d_in = D.from_numpy(values)
+    d_out = D.zeros(1, values.dtype)
+    capi.reduce(d_in, d_out, op=op)
+    sync()
+    return d_out.numpy()[0]
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.uint32, np.uint64])
+@pytest.mark.parametrize("op", OPS)
+def test_reduce_integers_exact(dtype, op):
+    for n in ARRAY_SIZES + [4096, 100003, (1 << 20) + 7]:
+        note("reduce", np.dtype(dtype).name, op, n)
+        v = random_ints(dtype, n, seed=n)
+        assert gpu_reduce(v, op) == O.reduce(v, op=op), n
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", ARRAY_SIZES[:-1] + [1000])
+def test_reduce_reference_float_sequences_exact(dtype, n):
+    # ReductionExtensionTests.tt:41-106: small integers, every partial sum is
+    # exactly representable, so the result must equal the left fold exactly.
+    for start, step in [(0, 1), (1, 0)]:
+        seq = compute_sequence(dtype, start, step, n)
+        for op in OPS:
+            assert gpu_reduce(seq, op) == O.reduce(seq, op=op)
+
+
+@pytest.mark.parametrize("n", [1, 3, 1000, 65537, 1 << 22])
+def test_reduce_float32_add_tolerance(n):
+    # Contract: |gpu - float64 host sum| <= 1e-5 * |float64 host sum|.
+    v = datagen.normal_f32(n, seed=n)
+    exact = O.sum_f64(v)
+    got = float(gpu_reduce(v, capi.OP_ADD))
+    note("reduce f32 add", n, got, exact)
+    # one float32 rounding of the exact sum is allowed on top
+    assert abs(got - exact) <= 1e-5 * abs(exact) + abs(exact) * 2.0 ** -24
+
+
+def test_reduce_float64_add_tolerance():
+    v = np.random.default_rng(1).standard_normal(1 << 20)
+    exact = O.sum_f64(v)
+    assert abs(float(gpu_reduce(v, capi.OP_ADD)) - exact) <= 1e-10 * max(1.0, abs(exact))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_reduce_float_max_min_semantics(dtype):
+    v = np.random.default_rng(2).standard_normal(50000).astype(dtype)
+    assert gpu_reduce(v, capi.OP_MAX) == v.max()
+    assert gpu_reduce(v, capi.OP_MIN) == v.min()
+    w = v.copy()
+    w[12345] = np.nan  # Math.Max/Min propagate NaN
+    assert np.isnan(gpu_reduce(w, capi.OP_MAX)) and np.isnan(gpu_reduce(w, capi.OP_MIN))
+    z = np.array([0.0, -0.0, 0.0], dtype=dtype)
+    assert np.signbit(gpu_reduce(z, capi.OP_MIN))
+    assert not np.signbit(gpu_reduce(z, capi.OP_MAX))
+    neg = np.full(100, -5.0, dtype=dtype)
+    assert gpu_reduce(neg, capi.OP_MAX) == -5.0
+
+
+def test_reduce_overwrites_output_and_accepts_unaligned_views():
+    v = random_ints(np.int32, 10000, seed=3)
+    d_all = D.from_numpy(v)
+    for off, n in [(1, 9999), (3, 5), (2, 4097), (5, 1)]:
+        d_out = D.from_numpy(np.array([12345, 777], dtype=np.int32))
+        capi.reduce(d_all.subview(off, n), d_out)
+        sync()
+        out = d_out.numpy()
+        with np.errstate(over="ignore"):
+            assert out[0] == np.sum(v[off:off + n], dtype=np.int32)
+        assert out[1] == 777  # only output[0] is written (ReductionExtensions.cs:156)
+
+
+# --------------------------------------------------------------------- scan
+def gpu_scan(values, op, inclusive, out_extra=0):
+    d_in = D.from_numpy(values)
+    d_out = D.from_numpy(np.full(values.size + out_extra, 77, dtype=values.dtype))
+    capi.scan(d_in, d_out, op=op,
+              kind=capi.SCAN_INCLUSIVE if inclusive else capi.SCAN_EXCLUSIVE)
+    sync()
+    return d_out.numpy()
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.uint32, np.uint64])
+@pytest.mark.parametrize("op", OPS)
+@pytest.mark.parametrize("inclusive", [True, False])
+def test_scan_integers_exact(dtype, op, inclusive):
+    for n in ARRAY_SIZES + [2048, 4095, 4096, 4097, 100003, (1 << 20) + 13]:
+        note("scan", np.dtype(dtype).name, op, inclusive, n)
+        v = random_ints(dtype, n, seed=n)
+        got = gpu_scan(v, op, inclusive)
+        assert np.array_equal(got, O.scan(v, op=op, inclusive=inclusive)), n
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("inclusive", [True, False])
+def test_scan_reference_float_sequences_exact(dtype, inclusive):
+    # ScanExtensionTests.tt:43-104 (floats up to 1000 elements): all partial
+    # results are exactly representable, so equality is exact.
+    for n in [1, 31, 33, 127, 1000]:
+        for start, step in [(0, 1), (1, 0), (n, -1)]:
+            seq = compute_sequence(dtype, start, step, n)
+            for op in OPS:
+                got = gpu_scan(seq, op, inclusive)
+                assert np.array_equal(got, O.scan(seq, op=op, inclusive=inclusive))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_scan_float_add_tolerance(dtype):
+    # The association order differs from the reference's 16-wide group scan;
+    # tolerance: 1e-5 (f32) / 1e-12 (f64) of the running sum of |x|.
+    n = 200003
+    v = np.random.default_rng(5).standard_normal(n).astype(dtype)
+    exact = np.cumsum(v.astype(np.float64))
+    scale = np.cumsum(np.abs(v.astype(np.float64)))
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    got = gpu_scan(v, capi.OP_ADD, True).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= tol * scale + 1e-30)
+    got = gpu_scan(v, capi.OP_ADD, False).astype(np.float64)
+    assert got[0] == 0.0
+    assert np.all(np.abs(got[1:] - exact[:-1]) <= tol * scale[:-1] + 1e-30)
+    assert np.array_equal(gpu_scan(v, capi.OP_MAX, True), np.maximum.accumulate(v))
+    assert np.array_equal(gpu_scan(v, capi.OP_MIN, True), np.minimum.accumulate(v))
+
+
+def test_scan_longer_output_in_place_and_unaligned_views():
+    v = random_ints(np.int32, 50000, seed=8)
+    with np.errstate(over="ignore"):
+        inc = np.cumsum(v, dtype=np.int32)
+    # output longer than input: only the first n are written (ScanExtensions.cs:679)
+    got = gpu_scan(v, capi.OP_ADD, True, out_extra=5)
+    assert np.array_equal(got[:-5], inc) and np.all(got[-5:] == 77)
+    # in place
+    d = D.from_numpy(v)
+    capi.scan(d, d)
+    sync()
+    assert np.array_equal(d.numpy(), inc)
+    # element-aligned but not 16-byte aligned views
+    d_in = D.from_numpy(v)
+    d_out = D.zeros(v.size, np.int32)
+    for off, n in [(1, 40001), (3, 4096), (2, 7)]:
+        capi.scan(d_in.subview(off, n), d_out.subview(1, n), kind=capi.SCAN_EXCLUSIVE)
+        sync()
+        with np.errstate(over="ignore"):
+            e = np.concatenate([[0], np.cumsum(v[off:off + n], dtype=np.int32)[:-1]])
+        assert np.array_equal(d_out.numpy()[1:1 + n], e.astype(np.int32))
+
+
+def test_scan_temp_buffer_can_be_reused_dirty():
+    v = datagen.small_ints_i32(300000, seed=1)
+    d_in, d_out = D.from_numpy(v), D.zeros(v.size, np.int32)
+    temp = capi.temp_buffer(capi.scan_temp_bytes(v.size, np.int32))
+    temp.bytes.fill_(0xFF)
+    for _ in range(3):
+        capi.scan(d_in, d_out, temp, kind=capi.SCAN_EXCLUSIVE)
+        sync()
+        assert np.array_equal(d_out.numpy(), O.scan(v, inclusive=False))
+
+
+# ---------------------------------------------------------------- histogram
+HIST_IN_DTYPES = [np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16,
+                  np.uint32, np.uint64, np.float32, np.float64]
+HIST_BIN_DTYPES = [np.int32, np.int64, np.uint32, np.uint64]
+
+
+def gpu_histogram(values, bins, locator, overflow=0, checked=True):
+    d_in, d_bins = D.from_numpy(values), D.from_numpy(bins)
+    d_ov = D.from_numpy(np.array([overflow], dtype=np.int32))
+    capi.histogram(d_in, d_bins, d_ov if checked else None, locator=locator)
+    sync()
+    return d_bins.numpy(), int(d_ov.numpy()[0])
+
+
+@pytest.mark.parametrize("in_dtype", HIST_IN_DTYPES)
+@pytest.mark.parametrize("bin_dtype", HIST_BIN_DTYPES)
+def test_histogram_reference_cases(in_dtype, bin_dtype):
+    # HistogramTests.tt:99-144 and :146-203.
+    values = np.arange(1, 1025).astype(in_dtype)
+    for num_bins in (64, 256):
+        zero = np.zeros(num_bins, dtype=bin_dtype)
+        assert_hist_equal(values, zero, capi.LOCATOR_MODULO)
+    info = np.iinfo(bin_dtype)
+    small = np.arange(1, 33).astype(in_dtype)
+    start = np.array([info.max - 32 - 1], dtype=bin_dtype)
+    bins1, ov1 = gpu_histogram(small, start, capi.LOCATOR_MODULO)
+    e1, eo1 = O.histogram(small, start, locator=O.LOCATOR_MODULO)
+    assert np.array_equal(bins1, e1) and ov1 == eo1 == 0
+    bins2, ov2 = gpu_histogram(small, bins1, capi.LOCATOR_MODULO)
+    e2, eo2 = O.histogram(small, e1, locator=O.LOCATOR_MODULO)
+    assert np.array_equal(bins2, e2) and ov2 == eo2 == 1
+
+
+def assert_hist_equal(values, bins, locator, overflow=0):
+    got, ov = gpu_histogram(values, bins, locator, overflow)
+    exp, eov = O.histogram(values, bins, locator=locator, overflow=overflow)
+    assert np.array_equal(got, exp)
+    assert ov == eov
+
+
+@pytest.mark.parametrize("n", [1, 100, 4099, (1 << 20) + 3])
+def test_histogram_bytes_256_bins(n):
+    note("hist u8", n)
+    v = datagen.bytes_u8(n, seed=n)
+    pre = random_ints(np.int32, 256, seed=1, lo=0, hi=1000)
+    assert_hist_equal(v, pre, capi.LOCATOR_IDENTITY)
+    # skew: a constant input hits one bin
+    assert_hist_equal(np.full(n, 200, dtype=np.uint8), pre, capi.LOCATOR_IDENTITY)
+
+
+@pytest.mark.parametrize("n", [1000, (1 << 20) + 5])
+def test_histogram_4096_bins_gaussian_mixture(n):
+    v = datagen.gaussian_mixture_i32(n, seed=n)
+    assert v.min() >= 0 and v.max() <= 4095
+    assert_hist_equal(v, np.zeros(4096, dtype=np.int32), capi.LOCATOR_IDENTITY)
+    assert_hist_equal(v, np.zeros(4096, dtype=np.uint64), capi.LOCATOR_IDENTITY)
+
+
+def test_histogram_many_bins_uses_global_atomics():
+    n, bins = 200000, 100000
+    v = random_ints(np.int32, n, seed=4, lo=0, hi=bins - 1)
+    assert_hist_equal(v, np.zeros(bins, dtype=np.int32), capi.LOCATOR_IDENTITY)
+    w = random_ints(np.int64, n, seed=5)
+    assert_hist_equal(w, np.zeros(bins, dtype=np.uint32), capi.LOCATOR_MODULO)
+
+
+def test_histogram_modulo_negative_and_wide_inputs():
+    for dtype in (np.int8, np.int32, np.int64, np.uint64):
+        v = random_ints(dtype, 30000, seed=6)
+        assert_hist_equal(v, np.zeros(100, dtype=np.int32), capi.LOCATOR_MODULO)
+    f = (np.random.default_rng(7).standard_normal(30000) * 1000).astype(np.float32)
+    assert_hist_equal(f, np.zeros(64, dtype=np.int32), capi.LOCATOR_MODULO)
+
+
+def test_histogram_identity_ignores_out_of_range_and_unchecked_variant():
+    v = np.array([-1, 0, 5, 256, 1000, 255, 255], dtype=np.int32)
+    got, ov = gpu_histogram(v, np.zeros(256, dtype=np.int32), capi.LOCATOR_IDENTITY)
+    exp = np.zeros(256, dtype=np.int32)
+    exp[0], exp[5], exp[255] = 1, 1, 2
+    assert np.array_equal(got, exp) and ov == 0
+    # HistogramUnchecked: no overflow word at all
+    start = np.array([np.iinfo(np.int32).max], dtype=np.int32)
+    got, ov = gpu_histogram(np.zeros(4, dtype=np.int32), start,
+                            capi.LOCATOR_IDENTITY, checked=False)
+    assert got[0] == np.int32(np.iinfo(np.int32).min + 3) and ov == 0
+    # the overflow word is OR-ed into
+    _, ov = gpu_histogram(np.zeros(4, dtype=np.int32), np.zeros(1, dtype=np.int32),
+                          capi.LOCATOR_IDENTITY, overflow=1)
+    assert ov == 1
+
+
+# --------------------------------------------------------------- radix sort
+def gpu_sort(keys, **kw):
+    d = D.from_numpy(keys)
+    capi.radix_sort_keys(d, **kw)
+    sync()
+    return d.numpy()
+
+
+def gpu_sort_pairs(keys, values, **kw):
+    dk, dv = D.from_numpy(keys), D.from_numpy(values)
+    capi.radix_sort_pairs(dk, dv, **kw)
+    sync()
+    return dk.numpy(), dv.numpy()
+
+
+def bits_equal(a, b):
+    return np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+@pytest.mark.parametrize("dtype", ATOMIC_NUMERIC_DTYPES)
+def test_sort_reference_cases(dtype):
+    # RadixSortExtensionTests.tt:144-230, 370-432.
+    for n in ARRAY_SIZES:
+        note("sort ref", np.dtype(dtype).name, n)
+        seq = compute_sequence(dtype, 0, 1, n)
+        inv = compute_inverted_sequence(dtype, 0, 1, n)
+        assert bits_equal(gpu_sort(inv), seq)
+        assert bits_equal(gpu_sort(seq), seq)
+        assert bits_equal(gpu_sort(seq, descending=True), inv)
+        assert bits_equal(gpu_sort(inv, descending=True), inv)
+        for start in (0, 1, -1):
+            if np.dtype(dtype).kind == "u" and start < 0:
+                continue
+            const = compute_sequence(dtype, start, 0, n)
+            assert bits_equal(gpu_sort(const), const)
+        k, v = gpu_sort_pairs(inv, inv)  # :319-365, values == keys
+        assert bits_equal(k, seq) and bits_equal(v, seq)
+
+
+def test_sort_2pow20_uniform_u32_bit_exact():
+    # Baseline config: 2^20 uniform uint32 keys, compared with the CPU path.
+    keys = datagen.uniform_u32(1 << 20)
+    assert np.array_equal(gpu_sort(keys), O.radix_sort(keys))
+
+
+@pytest.mark.parametrize("dtype", INT_KEY_DTYPES)
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_integer_types_match_oracle(dtype, descending):
+    for n in [1, 63, 64, 65, 4095, 4096, 4097, 8191, 8192, 8193, 50001]:
+        note("sort", np.dtype(dtype).name, descending, n)
+        keys = random_ints(dtype, n, seed=n)
+        assert np.array_equal(gpu_sort(keys, descending=descending),
+                              O.radix_sort(keys, descending=descending)), n
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_float_types_match_reference_order(dtype, descending):
+    # Default float order = the reference's ExtractRadixBits as written
+    # (parity unpinned by reference tests for negative values; see the oracle).
+    keys = random_float_bits(dtype, 30011, seed=3)
+    assert bits_equal(gpu_sort(keys, descending=descending),
+                      O.radix_sort(keys, descending=descending))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+def test_sort_float_total_order_flag(dtype):
+    # Extension without a reference counterpart: IEEE totalOrder.
+    keys = random_float_bits(dtype, 20000, seed=4)
+    u = {2: np.uint16, 4: np.uint32, 8: np.uint64}[np.dtype(dtype).itemsize]
+    bits = keys.view(u)
+    sign = u(1) << u(np.dtype(dtype).itemsize * 8 - 1)
+    ordered = np.where(bits & sign, ~bits, bits | sign)
+    expect = keys[np.argsort(ordered, kind="stable")]
+    assert bits_equal(gpu_sort(keys, float_total_order=True), expect)
+    assert bits_equal(gpu_sort(keys, float_total_order=True, descending=True),
+                      keys[np.argsort(~ordered, kind="stable")])
+
+
+@pytest.mark.parametrize("kind", ["zipf", "constant", "low16", "two_values"])
+def test_sort_skewed_inputs(kind):
+    n = (1 << 18) + 77
+    if kind == "zipf":
+        keys = datagen.zipf_u32(n)
+    elif kind == "constant":
+        keys = datagen.constant_u32(n)
+    elif kind == "low16":
+        keys = datagen.uniform_u32(n) & np.uint32(0xFFFF)
+    else:
+        keys = np.where(datagen.uniform_u32(n) & 1, np.uint32(0xFFFFFFFF), np.uint32(0))
+    assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+    values = np.arange(n, dtype=np.uint32)
+    k, v = gpu_sort_pairs(keys, values)
+    perm = np.argsort(keys, kind="stable")
+    assert np.array_equal(k, keys[perm]) and np.array_equal(v, values[perm])
+
+
+@pytest.mark.parametrize("key_dtype,value_dtype", [
+    (np.uint32, np.uint32), (np.uint64, np.uint32), (np.int32, np.float64),
+    (np.uint8, np.uint16), (np.int16, np.uint8), (np.uint64, np.uint64),
+    (np.float32, np.int32)])
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_pairs_stable_and_bit_exact(key_dtype, value_dtype, descending):
+    for n in [1, 100, 8193, 70001]:
+        note("pairs", np.dtype(key_dtype).name, np.dtype(value_dtype).name, n)
+        if np.dtype(key_dtype).kind == "f":
+            keys = np.abs(np.random.default_rng(n).integers(0, 50, n)).astype(key_dtype)
+        else:
+            keys = random_ints(key_dtype, n, seed=n, lo=0, hi=40)  # many ties
+        values = np.arange(n).astype(value_dtype)
+        k, v = gpu_sort_pairs(keys, values, descending=descending)
+        ek, ev = O.radix_sort_pairs(keys, values, descending=descending)
+        assert bits_equal(k, ek) and bits_equal(v, ev), n
+
+
+def test_sort_pairs_16_byte_values():
+    n = 20001
+    keys = random_ints(np.uint32, n, seed=1, lo=0, hi=1000)
+    values = np.zeros((n, 2), dtype=np.uint64)
+    values[:, 0] = np.arange(n)
+    values[:, 1] = ~np.arange(n, dtype=np.uint64)
+    dk = D.from_numpy(keys)
+    dv = D(n, np.dtype([("a", np.uint64), ("b", np.uint64)]),
+           _bytes=D.from_numpy(values.reshape(-1)).bytes)
+    temp = capi.temp_buffer(capi.radix_sort_temp_bytes(n, np.uint32, 16))
+    capi.check(capi.lib().ilgpu_hip_radix_sort_pairs(
+        None, dk.ptr, 1, dv.ptr, 1, n, capi.U32, 16, 0, capi.VALUES_FROM_VIEW,
+        temp.ptr, temp.nbytes))
+    sync()
+    perm = np.argsort(keys, kind="stable")
+    assert np.array_equal(dk.numpy(), keys[perm])
+    got = dv.bytes.cpu().numpy().view(np.uint64).reshape(n, 2)
+    assert np.array_equal(got, values[perm])
+
+
+@pytest.mark.parametrize("value_dtype", [np.uint32, np.int64])
+def test_sort_pairs_values_from_index(value_dtype):
+    # Sequencer form (RadixSortExtensions.cs:1017-1074 with Int32Sequencer /
+    # Int64Sequencer): value[i] = i, whatever the values view held before.
+    for keys in (datagen.uniform_u64(100003), datagen.constant_u32(5000),
+                 datagen.uniform_u32(9000) & np.uint32(0xFF)):
+        n = keys.size
+        dk = D.from_numpy(keys)
+        dv = D.from_numpy(np.full(n, 99, dtype=value_dtype))
+        capi.radix_sort_pairs(dk, dv, values_from_index=True)
+        sync()
+        perm = np.argsort(keys, kind="stable")
+        assert np.array_equal(dk.numpy(), keys[perm])
+        assert np.array_equal(dv.numpy(), perm.astype(value_dtype))
+
+
+def test_sort_reuses_dirty_temp_and_unaligned_key_view():
+    keys = datagen.uniform_u32(100001, seed=5)
+    temp = capi.temp_buffer(capi.radix_sort_temp_bytes(keys.size, np.uint32))
+    temp.bytes.fill_(0xAB)
+    for _ in range(2):
+        d = D.from_numpy(keys)
+        capi.radix_sort_keys(d, temp)
+        sync()
+        assert np.array_equal(d.numpy(), np.sort(keys))
+    d = D.from_numpy(keys)
+    view = d.subview(3, 50000)
+    capi.radix_sort_keys(view)
+    sync()
+    out = d.numpy()
+    assert np.array_equal(out[3:50003], np.sort(keys[3:50003]))
+    assert np.array_equal(out[:3], keys[:3]) and np.array_equal(out[50003:], keys[50003:])
