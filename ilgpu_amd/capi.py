@@ -34,7 +34,8 @@ LOCATOR_IDENTITY, LOCATOR_MODULO = 0, 1
 
 EXPORTS = [
     "ilgpu_hip_version", "ilgpu_hip_status_string",
-    "ilgpu_hip_last_runtime_error", "ilgpu_hip_radix_sort_temp_bytes",
+    "ilgpu_hip_last_runtime_error", "ilgpu_hip_profile_enable",
+    "ilgpu_hip_profile_query", "ilgpu_hip_radix_sort_temp_bytes",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
@@ -106,6 +107,11 @@ def lib() -> ctypes.CDLL:
         L.ilgpu_hip_status_string.argtypes = [i32]
         L.ilgpu_hip_status_string.restype = ctypes.c_char_p
         L.ilgpu_hip_last_runtime_error.restype = i32
+        L.ilgpu_hip_profile_enable.argtypes = [i32]
+        L.ilgpu_hip_profile_enable.restype = i32
+        L.ilgpu_hip_profile_query.argtypes = [
+            ctypes.c_char_p, p64, ctypes.POINTER(ctypes.c_double)]
+        L.ilgpu_hip_profile_query.restype = i32
         L.ilgpu_hip_radix_sort_temp_bytes.argtypes = [i64, i32, i32, p64]
         L.ilgpu_hip_radix_sort_keys.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64]
         L.ilgpu_hip_radix_sort_pairs.argtypes = [
@@ -123,6 +129,20 @@ def lib() -> ctypes.CDLL:
                 getattr(L, name).restype = i32
         _lib = L
     return _lib
+
+
+def profile_enable(enabled: bool) -> None:
+    """Switches per-kernel event timing on (clearing totals) or off."""
+    check(lib().ilgpu_hip_profile_enable(1 if enabled else 0))
+
+
+def profile_query(kernel_name: str):
+    """(launches, total milliseconds) of the named kernel since enabling."""
+    launches, total = ctypes.c_int64(0), ctypes.c_double(0.0)
+    check(lib().ilgpu_hip_profile_query(kernel_name.encode(),
+                                        ctypes.byref(launches),
+                                        ctypes.byref(total)))
+    return launches.value, total.value
 
 
 def status_string(status: int) -> str:

@@ -3,6 +3,10 @@
 // dispatch to the kernel launchers.  No GPU work is enqueued when validation
 // fails, and nothing here allocates device memory.
 #include <atomic>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
 
 #include "kernels.hpp"
 
@@ -26,6 +30,70 @@ int device_cu_count() {
     cus = 256;
   g_cu_count.store(cus, std::memory_order_relaxed);
   return cus;
+}
+
+// ---- per-kernel timing ------------------------------------------------------
+namespace {
+struct ProfileRecord {
+  const char* name;
+  hipEvent_t start, stop;
+};
+struct ProfileTotal {
+  std::string name;
+  int64_t launches;
+  double total_ms;
+};
+std::atomic<bool> g_profiling{false};
+std::mutex g_profile_mutex;
+std::vector<ProfileRecord> g_profile_pending;
+std::vector<ProfileTotal> g_profile_totals;
+
+// Waits for every pending event pair and folds it into the totals.
+void drain_profile_records() {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  for (const ProfileRecord& r : g_profile_pending) {
+    float ms = 0.0f;
+    if (hipEventSynchronize(r.stop) == hipSuccess &&
+        hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+      ProfileTotal* t = nullptr;
+      for (ProfileTotal& c : g_profile_totals)
+        if (c.name == r.name) t = &c;
+      if (t == nullptr) {
+        g_profile_totals.push_back({r.name, 0, 0.0});
+        t = &g_profile_totals.back();
+      }
+      t->launches += 1;
+      t->total_ms += ms;
+    }
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_profile_pending.clear();
+}
+}  // namespace
+
+ProfileScope::ProfileScope(hipStream_t stream, const char* name)
+    : stream_(stream), name_(name), start_(nullptr), active_(false) {
+  if (!g_profiling.load(std::memory_order_relaxed)) return;
+  if (hipEventCreate(&start_) != hipSuccess) return;
+  if (hipEventRecord(start_, stream_) != hipSuccess) {
+    (void)hipEventDestroy(start_);
+    return;
+  }
+  active_ = true;
+}
+
+ProfileScope::~ProfileScope() {
+  if (!active_) return;
+  hipEvent_t stop = nullptr;
+  if (hipEventCreate(&stop) != hipSuccess ||
+      hipEventRecord(stop, stream_) != hipSuccess) {
+    (void)hipEventDestroy(start_);
+    if (stop) (void)hipEventDestroy(stop);
+    return;
+  }
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  g_profile_pending.push_back({name_, start_, stop});
 }
 
 namespace {
@@ -82,6 +150,32 @@ const char* ilgpu_hip_status_string(int32_t status) {
 }
 
 int32_t ilgpu_hip_last_runtime_error(void) { return g_last_runtime_error; }
+
+int32_t ilgpu_hip_profile_enable(int32_t enabled) {
+  drain_profile_records();
+  if (enabled) {
+    std::lock_guard<std::mutex> lock(g_profile_mutex);
+    g_profile_totals.clear();
+  }
+  g_profiling.store(enabled != 0, std::memory_order_relaxed);
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t ilgpu_hip_profile_query(const char* kernel_name, int64_t* launches,
+                                double* total_ms) {
+  if (kernel_name == nullptr || launches == nullptr || total_ms == nullptr)
+    return ILGPU_HIP_ERROR_NULL_VIEW;
+  drain_profile_records();
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  *launches = 0;
+  *total_ms = 0.0;
+  for (const ProfileTotal& t : g_profile_totals)
+    if (t.name == kernel_name) {
+      *launches = t.launches;
+      *total_ms = t.total_ms;
+    }
+  return ILGPU_HIP_SUCCESS;
+}
 
 /* ---- radix sort -------------------------------------------------------- */
 

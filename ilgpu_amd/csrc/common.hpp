@@ -29,6 +29,25 @@ inline int64_t div_up(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Number of compute units of the current device (cached per process).
 int device_cu_count();
 
+// Optional per-kernel timing (the library's counterpart of ILGPU's
+// ProfilingMarker, ProfilingMarker.cs:19-61): while enabled through
+// ilgpu_hip_profile_enable(), every ProfileScope brackets its kernel launch
+// with a pair of HIP events on the launch stream.  Off by default; when off a
+// scope costs one relaxed atomic load.
+class ProfileScope {
+ public:
+  ProfileScope(hipStream_t stream, const char* name);
+  ~ProfileScope();
+  ProfileScope(const ProfileScope&) = delete;
+  ProfileScope& operator=(const ProfileScope&) = delete;
+
+ private:
+  hipStream_t stream_;
+  const char* name_;
+  hipEvent_t start_;
+  bool active_;
+};
+
 inline int elem_size(int32_t type) {
   switch (type) {
     case ILGPU_HIP_I8: case ILGPU_HIP_U8: return 1;

@@ -238,6 +238,7 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* bins,
                      int64_t num_bins, int32_t bin_type, int32_t* overflow) {
   const T* src = static_cast<const T*>(in);
   const int cus = device_cu_count();
+  ProfileScope scope(stream, "histogram");
   if (num_bins > kLdsBudgetWords) {
     int64_t blocks = div_up(n, kBlock);
     if (blocks > (int64_t)cus * 4) blocks = (int64_t)cus * 4;

@@ -514,13 +514,17 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
     int64_t blocks = div_up(div_up(a.n, Vec16<K>::N), kHistBlock);
     if (blocks > (int64_t)cus * 4) blocks = (int64_t)cus * 4;
     if (blocks < 1) blocks = 1;
+    ProfileScope scope(stream, "sort_histogram");
     hipLaunchKernelGGL((sort_histogram_kernel<K>), dim3((unsigned)blocks),
                        dim3(kHistBlock), lds, stream, keys_a, a.n, xf, passes,
                        shift, hist);
     ILGPU_HIP_CHECK(hipGetLastError());
   }
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(kRadix), 0, stream, hist, excl,
-                     plan, passes, (uint32_t)a.n);
+  {
+    ProfileScope scope(stream, "sort_plan");
+    hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(kRadix), 0, stream, hist, excl,
+                       plan, passes, (uint32_t)a.n);
+  }
   ILGPU_HIP_CHECK(hipGetLastError());
 
   int per_cu = 0;
@@ -532,15 +536,19 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   for (int p = 0; p < passes; ++p) {
     uint32_t* status =
         reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
-    hipLaunchKernelGGL((onesweep_kernel<KEY_BYTES, VALUE_BYTES>),
-                       dim3((unsigned)grid), dim3(kSortBlock), 0, stream,
-                       keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl, status,
-                       tickets + p, plan, (int)L.tiles, from_index);
+    {
+      ProfileScope scope(stream, "sort_onesweep");
+      hipLaunchKernelGGL((onesweep_kernel<KEY_BYTES, VALUE_BYTES>),
+                         dim3((unsigned)grid), dim3(kSortBlock), 0, stream,
+                         keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
+                         status, tickets + p, plan, (int)L.tiles, from_index);
+    }
     ILGPU_HIP_CHECK(hipGetLastError());
   }
   {
     int64_t blocks = div_up(a.n, 256);
     if (blocks > (int64_t)cus * 8) blocks = (int64_t)cus * 8;
+    ProfileScope scope(stream, "sort_finish");
     hipLaunchKernelGGL((finish_kernel<KEY_BYTES, VALUE_BYTES>),
                        dim3((unsigned)blocks), dim3(256), 0, stream, keys_a,
                        keys_b, vals_a, vals_b, a.n, plan, from_index);

@@ -126,12 +126,18 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* out,
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
   if (blocks < 1) blocks = 1;
   A* partials = reinterpret_cast<A*>(align_up((int64_t)(uintptr_t)temp, 16));
-  hipLaunchKernelGGL((reduce_partials_kernel<T, OP>), dim3((unsigned)blocks),
-                     dim3(kBlock), 0, stream, static_cast<const T*>(in), n,
-                     partials);
+  {
+    ProfileScope scope(stream, "reduce_partials");
+    hipLaunchKernelGGL((reduce_partials_kernel<T, OP>), dim3((unsigned)blocks),
+                       dim3(kBlock), 0, stream, static_cast<const T*>(in), n,
+                       partials);
+  }
   ILGPU_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL((reduce_final_kernel<T, OP>), dim3(1), dim3(kBlock), 0,
-                     stream, partials, (int)blocks, static_cast<T*>(out));
+  {
+    ProfileScope scope(stream, "reduce_final");
+    hipLaunchKernelGGL((reduce_final_kernel<T, OP>), dim3(1), dim3(kBlock), 0,
+                       stream, partials, (int)blocks, static_cast<T*>(out));
+  }
   ILGPU_HIP_CHECK(hipGetLastError());
   return ILGPU_HIP_SUCCESS;
 }

@@ -297,6 +297,7 @@ int32_t launch_typed(hipStream_t stream, const void* in, void* out, int64_t n,
   const bool vector = (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
                       (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   const int inclusive = kind == ILGPU_HIP_SCAN_INCLUSIVE ? 1 : 0;
+  ProfileScope scope(stream, "scan");
   if (vector) {
     hipLaunchKernelGGL((scan_kernel<T, OP, true>), dim3((unsigned)tiles),
                        dim3(kBlock), 0, stream, static_cast<const T*>(in),
@@ -331,6 +332,7 @@ int32_t launch_zero_words(hipStream_t stream, uint32_t* words, int64_t count) {
   if (count <= 0) return ILGPU_HIP_SUCCESS;
   int64_t blocks = div_up(count, 256 * 4);
   if (blocks > 2048) blocks = 2048;
+  ProfileScope scope(stream, "zero_words");
   hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)blocks), dim3(256), 0,
                      stream, words, count);
   ILGPU_HIP_CHECK(hipGetLastError());

@@ -104,3 +104,107 @@ def gaussian_mixture_i32(n: int, bins: int = 4096, components: int = 8,
         v = np.rint(256.0 + 512.0 * comp + sigma * z)
         out[lo:hi] = np.clip(v, 0, bins - 1).astype(np.int32)
     return out
+
+
+# ---- the same streams generated on the GPU (torch int64 arithmetic) ---------
+# int64 multiplication and addition wrap like uint64, and a logical right shift
+# is an arithmetic one followed by a mask, so the bits equal the numpy version.
+def _as_i64(v: int) -> int:
+    v &= 0xFFFFFFFFFFFFFFFF
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+def splitmix64_torch(n: int, seed: int = DEFAULT_SEED, start: int = 0,
+                     device: str = "cuda:0"):
+    """x_start .. x_{start+n-1} as an int64 tensor holding the uint64 bits."""
+    import torch
+
+    def lsr(z, k):
+        return (z >> k) & ((1 << (64 - k)) - 1)
+
+    out = torch.empty(n, dtype=torch.int64, device=device)
+    chunk = 1 << 26
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        i = torch.arange(start + lo + 1, start + hi + 1, dtype=torch.int64,
+                         device=device)
+        z = i * _as_i64(int(_GAMMA)) + _as_i64(seed)
+        z = (z ^ lsr(z, 30)) * _as_i64(int(_M1))
+        z = (z ^ lsr(z, 27)) * _as_i64(int(_M2))
+        out[lo:hi] = z ^ lsr(z, 31)
+    return out
+
+
+def _unit_float64_torch(x):
+    import torch
+    return ((x >> 11) & ((1 << 53) - 1)).to(torch.float64) * (1.0 / 9007199254740992.0)
+
+
+def uniform_u32_torch(n: int, seed: int = DEFAULT_SEED, device: str = "cuda:0"):
+    """Bits of uniform_u32 as an int32 tensor."""
+    import torch
+    return splitmix64_torch(n, seed, device=device).to(torch.int32)
+
+
+def small_ints_i32_torch(n: int, seed: int = DEFAULT_SEED, device: str = "cuda:0"):
+    import torch
+    return (splitmix64_torch(n, seed, device=device) & 15).to(torch.int32)
+
+
+def bytes_u8_torch(n: int, seed: int = DEFAULT_SEED, device: str = "cuda:0"):
+    import torch
+    return splitmix64_torch((n + 7) // 8, seed, device=device).view(torch.uint8)[:n]
+
+
+def zipf_u32_torch(n: int, s: float = 1.1, distinct: int = 1 << 16,
+                   seed: int = DEFAULT_SEED, device: str = "cuda:0"):
+    """Bits of zipf_u32 as an int32 tensor (same table, same comparisons)."""
+    import torch
+    w = 1.0 / np.power(np.arange(1, distinct + 1, dtype=np.float64), s)
+    cdf = np.cumsum(w)
+    cdf /= cdf[-1]
+    table = torch.from_numpy(cdf).to(device)
+    out = torch.empty(n, dtype=torch.int32, device=device)
+    chunk = 1 << 26
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        u = _unit_float64_torch(splitmix64_torch(hi - lo, seed, start=lo, device=device))
+        r = torch.searchsorted(table, u, right=True).clamp_(max=distinct - 1)
+        out[lo:hi] = r.to(torch.int32)
+    return out
+
+
+def _box_muller_torch(x0, x1):
+    import torch
+    u0 = 1.0 - _unit_float64_torch(x0)
+    u1 = _unit_float64_torch(x1)
+    return torch.sqrt(-2.0 * torch.log(u0)) * torch.cos(2.0 * np.pi * u1)
+
+
+def normal_f32_torch(n: int, seed: int = DEFAULT_SEED, device: str = "cuda:0"):
+    """Same construction as normal_f32; log/cos may differ from numpy's in the
+    last float64 bit, so equality with the host version is not guaranteed."""
+    import torch
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    chunk = 1 << 25
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        x = splitmix64_torch(2 * (hi - lo), seed, start=2 * lo, device=device)
+        out[lo:hi] = _box_muller_torch(x[0::2], x[1::2]).to(torch.float32)
+    return out
+
+
+def gaussian_mixture_i32_torch(n: int, bins: int = 4096, components: int = 8,
+                               sigma: float = 96.0, seed: int = DEFAULT_SEED,
+                               device: str = "cuda:0"):
+    import torch
+    out = torch.empty(n, dtype=torch.int32, device=device)
+    chunk = 1 << 25
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        x = splitmix64_torch(3 * (hi - lo), seed, start=3 * lo, device=device)
+        comp = (x[0::3] & (components - 1)).to(torch.float64)
+        z = _box_muller_torch(x[1::3], x[2::3])
+        v = torch.round(256.0 + 512.0 * comp + sigma * z)
+        out[lo:hi] = v.clamp_(0, bins - 1).to(torch.int32)
+    return out

@@ -107,6 +107,19 @@ const char *ilgpu_hip_status_string(int32_t status);
 /* hipError_t of the most recent failing HIP call on the calling thread. */
 int32_t ilgpu_hip_last_runtime_error(void);
 
+/* Per-kernel timing, the library's counterpart of ILGPU's profiling markers
+ * (ProfilingMarker.cs:19-61, enabled by Context.Builder.Profiling(),
+ * Context.Builder.cs:315-319).  While enabled, each kernel launch is bracketed
+ * by a pair of HIP events on its stream.  Enabling clears earlier totals.
+ * ilgpu_hip_profile_query waits for the recorded events and returns how often
+ * the named kernel ran and its summed duration.  Kernel names: "zero_words",
+ * "reduce_partials", "reduce_final", "scan", "histogram", "sort_histogram",
+ * "sort_plan", "sort_onesweep", "sort_finish".  Not meant for concurrent use
+ * from several threads. */
+int32_t ilgpu_hip_profile_enable(int32_t enabled);
+int32_t ilgpu_hip_profile_query(const char *kernel_name, int64_t *launches,
+                                double *total_ms);
+
 /* ---- radix sort ---------------------------------------------------------
  * Replaces: RadixSort<T,TStride> delegates made by CreateRadixSort
  * (RadixSortExtensions.cs:37-42, 1130-1337), RadixSortPairs delegates made by
