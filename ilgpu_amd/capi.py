@@ -18,7 +18,11 @@ from typing import Optional
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libilgpu_hip_algorithms.so")
+# ILGPU_HIP_ALGORITHMS_LIB selects another build of the same library (e.g. one
+# compiled with different tuning constants); it must export the same C ABI.
+LIB_PATH = os.environ.get(
+    "ILGPU_HIP_ALGORITHMS_LIB",
+    os.path.join(_HERE, "lib", "libilgpu_hip_algorithms.so"))
 
 # ilgpu_hip_status
 SUCCESS, ERROR_NULL_VIEW, ERROR_OUT_OF_RANGE, ERROR_NOT_SUPPORTED, \

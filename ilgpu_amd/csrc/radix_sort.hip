@@ -14,8 +14,8 @@
 //             marks passes whose digit is the same for every key (they are
 //             skipped) and records which buffer each pass reads;
 //   pass x k  onesweep: a block takes a tile by ticket, ranks its keys
-//             (per-wave digit counters in LDS, wave64 ballot matching, so
-//             equal digits keep memory order: every pass is stable), publishes
+//             (per-half-wave {peer mask, count} slots in LDS, so equal digits
+//             keep memory order: every pass is stable), publishes
 //             its 256 digit counts, resolves the counts of all earlier tiles by
 //             decoupled look-back, stages the tile in digit order through LDS
 //             and writes each digit's run to its final place;
@@ -39,8 +39,23 @@ namespace {
 
 constexpr int kRadix = 256;
 constexpr int kMaxPasses = 8;
-constexpr int kSortBlock = 512;
-constexpr int kSortWaves = kSortBlock / kWaveSize;
+// Launch shape of the onesweep pass.  The block size fixes the number of
+// half-wave sub-tiles (and with it the LDS footprint of the ranking words);
+// items per thread fix the tile size.
+#ifndef ILGPU_HIP_SORT_BLOCK
+#define ILGPU_HIP_SORT_BLOCK 512
+#endif
+#ifndef ILGPU_HIP_SORT_ITEMS
+#define ILGPU_HIP_SORT_ITEMS 16
+#endif
+#ifndef ILGPU_HIP_SORT_WAVES_PER_EU
+#define ILGPU_HIP_SORT_WAVES_PER_EU 4
+#endif
+#ifndef ILGPU_HIP_SORT_LOOKBACK
+#define ILGPU_HIP_SORT_LOOKBACK 4
+#endif
+constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;
+constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
 constexpr int kHistBlock = 512;
 constexpr uint32_t kStatusAggregate = 1u << 30;
 constexpr uint32_t kStatusPrefix = 2u << 30;
@@ -61,7 +76,8 @@ template <> struct ValueOf<8> { using type = uint64_t; };
 template <> struct ValueOf<16> { using type = Bytes16; };
 
 template <int KEY_BYTES> constexpr int items_per_thread() {
-  return KEY_BYTES == 8 ? 8 : 16;
+  // 8-byte keys take two registers each: half the items, same bytes per tile.
+  return KEY_BYTES == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_ITEMS;
 }
 template <int KEY_BYTES> constexpr int tile_keys() {
   return kSortBlock * items_per_thread<KEY_BYTES>();
@@ -212,20 +228,261 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 }
 
 // ---- onesweep pass ---------------------------------------------------------
-// Lanes holding the same digit, as a 64-bit mask: eight ballots, one per bit.
-__device__ __forceinline__ uint64_t match_digit(uint32_t d) {
-  uint64_t peers = ~0ull;
+// Ranking.  A block's tile is cut into sub-tiles, one per half-wave (32
+// lanes); lane l of half-wave h holds items h*32*kItems + j*32 + l, j = 0 ..
+// kItems-1, so memory order inside a sub-tile is (row j, lane).  Every
+// (half-wave, digit) pair owns a peer-mask word and a running-count word in
+// LDS.  For row j every lane
+//   1. ORs its lane bit into the mask word of its digit (LDS atomic),
+//   2. reads mask and count back: the mask now names all lanes of the
+//      half-wave holding that digit in this row, the count is the number of
+//      keys with the digit in earlier rows,
+//   3. ranks itself: count + number of peers in lower lanes,
+//   4. and the lowest peer stores count + number of peers and clears the mask
+//      for the next row.
+// LDS instructions of one wave execute in issue order, so the rows chain
+// through the two words without barriers, and equal digits keep memory
+// order: the pass is stable.  No ballots: the cost per key is a handful of
+// LDS operations and about ten VALU operations whatever the key distribution.
+template <int KEY_BYTES> struct SortTile {
+  static constexpr int kSubTiles = kSortBlock / 32;
+  static constexpr int kSlotWords = kSubTiles * kRadix;      // per array
+  static constexpr int kSlotBytes = 2 * kSlotWords * 4;      // masks + counts
+  static constexpr int kItems = items_per_thread<KEY_BYTES>();
+  static constexpr int kTile = tile_keys<KEY_BYTES>();
+  static constexpr int kSubTileKeys = 32 * kItems;
+  static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
+  static constexpr int kStageBytes =
+      kSlotBytes > kKeyStageBytes ? kSlotBytes : kKeyStageBytes;
+};
+
+template <int KEY_BYTES, bool FULL>
+__device__ __forceinline__ void load_tile_keys(
+    const typename KeyOf<KEY_BYTES>::type* __restrict__ src, int64_t tile_base,
+    int valid, int first_local,
+    typename KeyOf<KEY_BYTES>::type (&key)[SortTile<KEY_BYTES>::kItems]) {
 #pragma unroll
-  for (int b = 0; b < 8; ++b) {
-    const bool bit = (d >> b) & 1u;
-    const uint64_t m = __ballot(bit);
-    peers &= bit ? m : ~m;
+  for (int j = 0; j < SortTile<KEY_BYTES>::kItems; ++j) {
+    const int local = first_local + j * 32;
+    if (FULL || local < valid) key[j] = src[tile_base + local];
+    else key[j] = 0;
   }
-  return peers;
 }
 
-template <int KEY_BYTES, int VALUE_BYTES>
-__global__ __launch_bounds__(kSortBlock) void onesweep_kernel(
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL>
+__device__ __forceinline__ void sort_tile(
+    typename KeyOf<KEY_BYTES>::type (&key)[SortTile<KEY_BYTES>::kItems],
+    typename KeyOf<KEY_BYTES>::type* __restrict__ dst_keys,
+    const typename ValueOf<VALUE_BYTES>::type* __restrict__ src_vals,
+    typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
+    int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
+    const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
+    unsigned char* s_stage, uint32_t* s_digit_start, uint32_t* s_global_off,
+    uint32_t* s_scan,
+    // Fetching the next tile: its ticket is drawn after this tile's look-back
+    // and its keys are loaded while this tile is staged and written out.
+    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int64_t n,
+    uint32_t* ticket, int num_tiles, int* s_next_tile, int& next_tile,
+    typename KeyOf<KEY_BYTES>::type (&next_key)[SortTile<KEY_BYTES>::kItems]) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  using Val = typename ValueOf<VALUE_BYTES>::type;
+  using TileCfg = SortTile<KEY_BYTES>;
+  constexpr int kItems = TileCfg::kItems;
+  constexpr int kSubTiles = TileCfg::kSubTiles;
+  constexpr int kSlotWords = TileCfg::kSlotWords;
+  constexpr bool kPairs = VALUE_BYTES > 0;
+  constexpr int kValuesPerRound =
+      kPairs ? TileCfg::kStageBytes / (VALUE_BYTES > 0 ? VALUE_BYTES : 1) : 1;
+  constexpr int kRounds =
+      kPairs ? (TileCfg::kTile + kValuesPerRound - 1) / kValuesPerRound : 0;
+
+  uint32_t* s_mask = reinterpret_cast<uint32_t*>(s_stage);
+  uint32_t* s_count = s_mask + kSlotWords;
+  K* s_keys = reinterpret_cast<K*>(s_stage);
+  Val* s_vals = reinterpret_cast<Val*>(s_stage);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int wave = tid / kWaveSize;
+  const int sub = tid >> 5;                 // half-wave index in the block
+  const int sub_lane = tid & 31;
+  const uint32_t lane_bit = 1u << sub_lane;
+  const uint32_t lower_lanes = lane_bit - 1u;
+  const int first_local = sub * TileCfg::kSubTileKeys + sub_lane;
+  const int shift = pass * 8;
+
+  auto digit = [&](K k) -> uint32_t {
+    if constexpr (FLOAT_KEYS) return digit_of(k, xf, shift);
+    else return (uint32_t)((K)(k ^ (K)xf.xor_mask) >> shift) & (kRadix - 1);
+  };
+
+  Val val[kPairs ? kItems : 1];
+  if constexpr (kPairs) {
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const int local = first_local + j * 32;
+      if (FULL || local < valid) {
+        if (make_index) {
+          if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)(tile_base + local);
+          else if constexpr (VALUE_BYTES == 8) val[j] = (Val)(uint64_t)(tile_base + local);
+        } else {
+          val[j] = src_vals[tile_base + local];
+        }
+      }
+    }
+  }
+
+  // Keys past the end of the input take digit 255; they come last in memory
+  // order, so they rank behind every real key and are dropped on write-out.
+  uint32_t* my_mask = s_mask + sub * kRadix;
+  uint32_t rank[kItems];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const int local = first_local + j * 32;
+    const uint32_t d = (FULL || local < valid) ? digit(key[j]) : (kRadix - 1);
+    uint32_t* mask_word = my_mask + d;
+    uint32_t* count_word = mask_word + kSlotWords;
+    __hip_atomic_fetch_or(mask_word, lane_bit, __ATOMIC_RELAXED,
+                          __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t peers = __hip_atomic_load(mask_word, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t before = __hip_atomic_load(count_word, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t below = (uint32_t)__popc(peers & lower_lanes);
+    if (below == 0) {
+      __hip_atomic_store(count_word, before + (uint32_t)__popc(peers),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_store(mask_word, 0u, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    rank[j] = before + below;
+  }
+  __syncthreads();
+
+  // One thread per digit: totals over the sub-tiles, look-back over the tiles.
+  uint32_t count = 0, inc = 0;
+  uint32_t* tile_status = status + (int64_t)tile * kRadix;
+  if (tid < kRadix) {
+#pragma unroll
+    for (int s = 0; s < kSubTiles; ++s) {
+      const uint32_t t = s_count[s * kRadix + tid];
+      s_count[s * kRadix + tid] = count;
+      count += t;
+    }
+    __hip_atomic_store(&tile_status[tid],
+                       (tile == 0 ? kStatusPrefix : kStatusAggregate) | count,
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    inc = count;
+#pragma unroll
+    for (int s = 1; s < kWaveSize; s <<= 1) {
+      const uint32_t o = shfl_up(inc, s);
+      if (lane >= s) inc += o;
+    }
+    if (lane == kWaveSize - 1) s_scan[wave] = inc;
+  }
+  __syncthreads();
+  if (tid < kRadix) {
+    uint32_t digit_start = inc - count;
+    for (int w = 0; w < wave; ++w) digit_start += s_scan[w];
+    s_digit_start[tid] = digit_start;
+
+    // Keys with this digit in earlier tiles: walk back over the status words,
+    // kLookback tiles per step.  The loads of a step are unconditional (index
+    // clamped) so that they are in flight together; positions in front of
+    // tile 0 read as an empty inclusive prefix.
+    uint32_t before = 0;
+    bool done = tile == 0;
+    for (int t = tile - 1; !done; t -= kLookback) {
+      uint32_t s[kLookback];
+#pragma unroll
+      for (int u = 0; u < kLookback; ++u) {
+        const int idx = t - u < 0 ? 0 : t - u;
+        s[u] = __hip_atomic_load(&status[(int64_t)idx * kRadix + tid],
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+      for (int u = 0; u < kLookback; ++u)
+        if (t - u < 0) s[u] = kStatusPrefix;
+#pragma unroll
+      for (int u = 0; u < kLookback; ++u) {
+        if (done) continue;
+        while ((s[u] & ~kStatusValueMask) == 0) {
+          __builtin_amdgcn_s_sleep(1);
+          s[u] = __hip_atomic_load(&status[(int64_t)(t - u) * kRadix + tid],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        before += s[u] & kStatusValueMask;
+        done = (s[u] & ~kStatusValueMask) == kStatusPrefix;
+      }
+    }
+    if (tile > 0)
+      __hip_atomic_store(&tile_status[tid], kStatusPrefix | (before + count),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_global_off[tid] = excl[pass * kRadix + tid] + before - digit_start;
+    if (tid == 0) *s_next_tile = (int)atomicAdd(ticket, 1u);
+  }
+  __syncthreads();
+  next_tile = *s_next_tile;
+  {
+    const int64_t next_base = (int64_t)next_tile * TileCfg::kTile;
+    const int64_t remaining = n - next_base;
+    if (next_tile < num_tiles && remaining >= TileCfg::kTile)
+      load_tile_keys<KEY_BYTES, true>(src_keys, next_base, TileCfg::kTile, first_local, next_key);
+    else
+      load_tile_keys<KEY_BYTES, false>(
+          src_keys, next_base,
+          next_tile < num_tiles && remaining > 0 ? (int)remaining : 0,
+          first_local, next_key);
+  }
+
+  // Tile-local position of every key; afterwards the mask/count words are
+  // dead and the same LDS bytes stage the keys in digit order.
+  uint32_t pos[kItems];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const int local = first_local + j * 32;
+    const uint32_t d = (FULL || local < valid) ? digit(key[j]) : (kRadix - 1);
+    pos[j] = s_count[sub * kRadix + d] + s_digit_start[d] + rank[j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) s_keys[pos[j]] = key[j];
+  __syncthreads();
+
+  uint32_t gpos[kPairs ? kItems : 1];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const int i = j * kSortBlock + tid;
+    if (FULL || i < valid) {
+      const K k = s_keys[i];
+      const uint32_t g = s_global_off[digit(k)] + (uint32_t)i;
+      dst_keys[g] = k;
+      if constexpr (kPairs) gpos[j] = g;
+    }
+  }
+
+  if constexpr (kPairs) {
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+      const uint32_t lo = (uint32_t)r * kValuesPerRound;
+      __syncthreads();  // the stage buffer is free again
+#pragma unroll
+      for (int j = 0; j < kItems; ++j)
+        if (pos[j] - lo < (uint32_t)kValuesPerRound) s_vals[pos[j] - lo] = val[j];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < kItems; ++j) {
+        const uint32_t i = (uint32_t)(j * kSortBlock + tid);
+        if ((FULL || i < (uint32_t)valid) && i - lo < (uint32_t)kValuesPerRound)
+          dst_vals[gpos[j]] = s_vals[i - lo];
+      }
+    }
+  }
+}
+
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS>
+__global__ __launch_bounds__(kSortBlock, ILGPU_HIP_SORT_WAVES_PER_EU)
+void onesweep_kernel(
     typename KeyOf<KEY_BYTES>::type* keys_a,
     typename KeyOf<KEY_BYTES>::type* keys_b,
     typename ValueOf<VALUE_BYTES>::type* vals_a,
@@ -235,21 +492,15 @@ __global__ __launch_bounds__(kSortBlock) void onesweep_kernel(
     int values_from_index) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  constexpr int kItems = items_per_thread<KEY_BYTES>();
-  constexpr int kTile = tile_keys<KEY_BYTES>();
-  constexpr bool kPairs = VALUE_BYTES > 0;
-  // Values are staged through the key buffer, kTile * KEY_BYTES bytes at a time.
-  constexpr int kStageBytes = kTile * (KEY_BYTES < 4 ? 4 : KEY_BYTES);
-  constexpr int kValuesPerRound = kPairs ? kStageBytes / (VALUE_BYTES > 0 ? VALUE_BYTES : 1) : 1;
-  constexpr int kRounds = kPairs ? (kTile + kValuesPerRound - 1) / kValuesPerRound : 0;
+  using TileCfg = SortTile<KEY_BYTES>;
+  constexpr int kTile = TileCfg::kTile;
+  constexpr int kItems = TileCfg::kItems;
 
-  __shared__ uint32_t s_wave_hist[kSortWaves][kRadix];
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[TileCfg::kStageBytes];
+  __shared__ uint32_t s_digit_start[kRadix];
   __shared__ uint32_t s_global_off[kRadix];
   __shared__ uint32_t s_scan[kRadix / kWaveSize];
-  __shared__ int s_tile;
-  __shared__ __attribute__((aligned(16))) unsigned char s_stage[kStageBytes];
-  K* s_keys = reinterpret_cast<K*>(s_stage);
-  Val* s_vals = reinterpret_cast<Val*>(s_stage);
+  __shared__ int s_tile[2];
 
   if (plan->skip[pass]) return;
   const bool src_alt = plan->src_is_alt[pass] != 0;
@@ -257,149 +508,50 @@ __global__ __launch_bounds__(kSortBlock) void onesweep_kernel(
   K* dst_keys = src_alt ? keys_a : keys_b;
   const Val* src_vals = src_alt ? vals_b : vals_a;
   Val* dst_vals = src_alt ? vals_a : vals_b;
-  const bool make_index = kPairs && values_from_index &&
+  const bool make_index = VALUE_BYTES > 0 && values_from_index &&
                           plan->first_executed == (uint32_t)pass;
-  const int shift = pass * 8;
   const int tid = threadIdx.x;
-  const int lane = tid & (kWaveSize - 1);
-  const int wave = tid / kWaveSize;
+  const int first_local = (tid >> 5) * TileCfg::kSubTileKeys + (tid & 31);
 
-  while (true) {
-    if (tid == 0) s_tile = (int)atomicAdd(ticket, 1u);
-    for (int i = tid; i < kSortWaves * kRadix; i += kSortBlock)
-      (&s_wave_hist[0][0])[i] = 0u;
+  auto valid_keys = [&](int t) -> int {
+    const int64_t remaining = n - (int64_t)t * kTile;
+    return remaining >= kTile ? kTile : (remaining > 0 ? (int)remaining : 0);
+  };
+
+  if (tid == 0) s_tile[0] = (int)atomicAdd(ticket, 1u);
+  __syncthreads();
+  int tile = s_tile[0];
+  K key[kItems];
+  if (tile < num_tiles) {
+    const int valid = valid_keys(tile);
+    if (valid == kTile) load_tile_keys<KEY_BYTES, true>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
+    else load_tile_keys<KEY_BYTES, false>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
+  }
+  while (tile < num_tiles) {
+    {  // clear the mask and count words
+      uint4* z = reinterpret_cast<uint4*>(s_stage);
+      for (int i = tid; i < TileCfg::kSlotBytes / 16; i += kSortBlock)
+        z[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
     __syncthreads();
-    const int tile = s_tile;
-    if (tile >= num_tiles) break;
-
     const int64_t tile_base = (int64_t)tile * kTile;
-    const int64_t remaining = n - tile_base;
-    const int valid = remaining < kTile ? (int)remaining : kTile;
-    const int wave_first = wave * (kWaveSize * kItems) + lane;
-
-    K key[kItems];
-    Val val[kPairs ? kItems : 1];
-#pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-      const int local = wave_first + j * kWaveSize;
-      if (local < valid) {
-        key[j] = src_keys[tile_base + local];
-        if constexpr (kPairs) {
-          if (make_index) {
-            if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)(tile_base + local);
-            else if constexpr (VALUE_BYTES == 8) val[j] = (Val)(uint64_t)(tile_base + local);
-          } else {
-            val[j] = src_vals[tile_base + local];
-          }
-        }
-      } else {
-        key[j] = 0;
-      }
+    const int valid = valid_keys(tile);
+    int next = num_tiles;
+    K next_key[kItems];
+    if (valid == kTile) {
+      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, true>(
+          key, dst_keys, src_vals, dst_vals, tile_base, kTile, tile, pass, xf,
+          excl, status, make_index, s_stage, s_digit_start, s_global_off, s_scan,
+          src_keys, n, ticket, num_tiles, &s_tile[1], next, next_key);
+    } else {
+      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false>(
+          key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
+          excl, status, make_index, s_stage, s_digit_start, s_global_off, s_scan,
+          src_keys, n, ticket, num_tiles, &s_tile[1], next, next_key);
     }
-
-    // Rank every key among the keys of its wave that share its digit; keys
-    // past the end of the input take digit 255 and, coming last in memory
-    // order, rank behind every real key.
-    uint32_t rank[kItems];
 #pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-      const int local = wave_first + j * kWaveSize;
-      const uint32_t d = local < valid ? digit_of(key[j], xf, shift) : (kRadix - 1);
-      const uint64_t peers = match_digit(d);
-      const uint32_t below = (uint32_t)mbcnt(peers);
-      const uint32_t prev = s_wave_hist[wave][d];
-      if (below == 0) s_wave_hist[wave][d] = prev + (uint32_t)__popcll(peers);
-      rank[j] = prev + below;
-    }
-    __syncthreads();
-
-    // One thread per digit: totals over the waves, look-back over the tiles.
-    uint32_t count = 0, inc = 0;
-    uint32_t* tile_status = status + (int64_t)tile * kRadix;
-    if (tid < kRadix) {
-#pragma unroll
-      for (int w = 0; w < kSortWaves; ++w) {
-        const uint32_t t = s_wave_hist[w][tid];
-        s_wave_hist[w][tid] = count;
-        count += t;
-      }
-      __hip_atomic_store(&tile_status[tid],
-                         (tile == 0 ? kStatusPrefix : kStatusAggregate) | count,
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      inc = count;
-#pragma unroll
-      for (int s = 1; s < kWaveSize; s <<= 1) {
-        const uint32_t o = shfl_up(inc, s);
-        if (lane >= s) inc += o;
-      }
-      if (lane == kWaveSize - 1) s_scan[wave] = inc;
-    }
-    __syncthreads();
-    if (tid < kRadix) {
-      uint32_t digit_start = inc - count;
-      for (int w = 0; w < wave; ++w) digit_start += s_scan[w];
-#pragma unroll
-      for (int w = 0; w < kSortWaves; ++w) s_wave_hist[w][tid] += digit_start;
-
-      uint32_t before = 0;  // keys with this digit in earlier tiles
-      for (int t = tile - 1; t >= 0; --t) {
-        uint32_t s;
-        while (true) {
-          s = __hip_atomic_load(&status[(int64_t)t * kRadix + tid],
-                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if ((s & ~kStatusValueMask) != 0) break;
-          __builtin_amdgcn_s_sleep(1);
-        }
-        before += s & kStatusValueMask;
-        if ((s & ~kStatusValueMask) == kStatusPrefix) break;
-      }
-      if (tile > 0)
-        __hip_atomic_store(&tile_status[tid], kStatusPrefix | (before + count),
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_global_off[tid] = excl[pass * kRadix + tid] + before - digit_start;
-    }
-    __syncthreads();
-
-    // Tile-local position of every key, then the keys in digit order in LDS.
-    uint32_t pos[kItems];
-#pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-      const int local = wave_first + j * kWaveSize;
-      const uint32_t d = local < valid ? digit_of(key[j], xf, shift) : (kRadix - 1);
-      pos[j] = s_wave_hist[wave][d] + rank[j];
-      s_keys[pos[j]] = key[j];
-    }
-    __syncthreads();
-
-    uint32_t gpos[kPairs ? kItems : 1];
-#pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-      const int i = j * kSortBlock + tid;
-      if (i < valid) {
-        const K k = s_keys[i];
-        const uint32_t g = s_global_off[digit_of(k, xf, shift)] + (uint32_t)i;
-        dst_keys[g] = k;
-        if constexpr (kPairs) gpos[j] = g;
-      }
-    }
-
-    if constexpr (kPairs) {
-#pragma unroll
-      for (int r = 0; r < kRounds; ++r) {
-        const uint32_t lo = (uint32_t)r * kValuesPerRound;
-        __syncthreads();  // the stage buffer is free again
-#pragma unroll
-        for (int j = 0; j < kItems; ++j)
-          if (pos[j] - lo < (uint32_t)kValuesPerRound) s_vals[pos[j] - lo] = val[j];
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < kItems; ++j) {
-          const uint32_t i = (uint32_t)(j * kSortBlock + tid);
-          if (i < (uint32_t)valid && i - lo < (uint32_t)kValuesPerRound)
-            dst_vals[gpos[j]] = s_vals[i - lo];
-        }
-      }
-    }
+    for (int j = 0; j < kItems; ++j) key[j] = next_key[j];
+    tile = next;
     __syncthreads();  // LDS is reused by the next tile
   }
 }
@@ -527,9 +679,14 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   }
   ILGPU_HIP_CHECK(hipGetLastError());
 
+  const bool float_keys = xf.mode != kModePlain;
+  auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false>;
+  if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
+    if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true>;
+  }
   int per_cu = 0;
   ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
-      &per_cu, onesweep_kernel<KEY_BYTES, VALUE_BYTES>, kSortBlock, 0));
+      &per_cu, pass_kernel, kSortBlock, 0));
   if (per_cu < 1) per_cu = 1;
   int64_t grid = (int64_t)cus * per_cu;
   if (grid > L.tiles) grid = L.tiles;
@@ -538,7 +695,7 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
         reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
     {
       ProfileScope scope(stream, "sort_onesweep");
-      hipLaunchKernelGGL((onesweep_kernel<KEY_BYTES, VALUE_BYTES>),
+      hipLaunchKernelGGL(pass_kernel,
                          dim3((unsigned)grid), dim3(kSortBlock), 0, stream,
                          keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
                          status, tickets + p, plan, (int)L.tiles, from_index);
