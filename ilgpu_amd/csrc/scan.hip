@@ -7,7 +7,9 @@
 // it, and a tile's first wave resolves the prefix of up to 64 predecessor
 // tiles per step, so tiles only wait for data, never for their turn.
 //
-// Tile layout (kBlock = 256 threads, 4 waves, kVecs 16-byte vectors per lane):
+// Tile layout (kBlock = 512 threads, 8 waves, kVecs = 16 16-byte vectors per
+// lane, i.e. 128 KiB per tile: time per launch falls with the number of tiles
+// until about this size, then register pressure takes over):
 //   wave w owns a contiguous chunk of kVecs*64 vectors; vector j of lane l is
 //   chunk[j*64 + l], so every load/store instruction of a wave covers 1 KiB of
 //   consecutive addresses (dwordx4 per lane).  Scan order inside a wave is
@@ -27,9 +29,15 @@ namespace ilgpu_hip {
 
 namespace {
 
-constexpr int kBlock = 256;
+#ifndef ILGPU_HIP_SCAN_BLOCK
+#define ILGPU_HIP_SCAN_BLOCK 512
+#endif
+#ifndef ILGPU_HIP_SCAN_VECS
+#define ILGPU_HIP_SCAN_VECS 16
+#endif
+constexpr int kBlock = ILGPU_HIP_SCAN_BLOCK;
 constexpr int kWaves = kBlock / kWaveSize;
-constexpr int kVecs = 4;
+constexpr int kVecs = ILGPU_HIP_SCAN_VECS;
 constexpr uint32_t kFlagInvalid = 0, kFlagAggregate = 1, kFlagPrefix = 2;
 constexpr int64_t kHeaderBytes = 256;  // ticket counter, padded
 
@@ -250,7 +258,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
       V v;
 #pragma unroll
       for (int k = 0; k < VN; ++k) v[k] = r[k];
-      dst[j * kWaveSize + lane] = v;
+      __builtin_nontemporal_store(v, &dst[j * kWaveSize + lane]);
     } else {
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
