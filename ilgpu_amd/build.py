@@ -62,5 +62,25 @@ def build(jobs: int | None = None) -> str:
     return LIB_PATH
 
 
+HOST_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp",
+                             "host_api_tests.cpp")
+HOST_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp",
+                             "host_api_tests")
+
+
+def build_host_example() -> str:
+    """Compiles the C++ host-layer test program against the built library."""
+    cmd = [HIPCC, "-x", "c++", "-std=c++17", "-O2", "-D__HIP_PLATFORM_AMD__",
+           "-I/opt/rocm/include", HOST_TEST_SRC, "-o", HOST_TEST_BIN,
+           "-L" + LIB_DIR, "-lilgpu_hip_algorithms",
+           "-L/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN/../../ilgpu_amd/lib", "-Wl,-rpath,/opt/rocm/lib"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"host test build failed:\n{proc.stderr}")
+    return HOST_TEST_BIN
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_host_example())

@@ -1,0 +1,381 @@
+// Tests of the C++ host layer, written after the reference's own suites
+// (ILGPU.Algorithms.Tests: RadixSortExtensionTests.tt, ScanExtensionTests.tt,
+// ReductionExtensionTests.tt, HistogramTests.tt, TempViewManagerTests.cs):
+// same sequences, sizes, call pattern (create once, invoke with a stream,
+// synchronise, verify) and expectations computed on the host.
+//
+//   host_api_tests            all tests (needs a GPU)
+//   host_api_tests --host     only the tests that touch no device
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../ilgpu_amd/host/ilgpu_hip_algorithms.hpp"
+
+using namespace ilgpu;
+using namespace ilgpu::Algorithms;
+namespace RSO = ilgpu::RadixSortOperations;
+namespace SRO = ilgpu::ScanReduceOperations;
+
+static int g_failed = 0, g_run = 0;
+#define CHECK(cond)                                                            \
+  do {                                                                         \
+    if (!(cond)) {                                                             \
+      std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);          \
+      ++g_failed;                                                              \
+    }                                                                          \
+  } while (0)
+#define EXPECT_THROW(stmt, Ex)                                                 \
+  do {                                                                         \
+    bool caught = false;                                                       \
+    try { stmt; } catch (const Ex&) { caught = true; } catch (...) {}          \
+    if (!caught) {                                                             \
+      std::printf("  FAILED %s:%d: expected %s\n", __FILE__, __LINE__, #Ex);   \
+      ++g_failed;                                                              \
+    }                                                                          \
+  } while (0)
+#define RUN(fn)                                                                \
+  do {                                                                         \
+    std::printf("[ RUN  ] %s\n", #fn);                                         \
+    std::fflush(stdout);                                                       \
+    ++g_run;                                                                   \
+    fn;                                                                        \
+  } while (0)
+
+// ArraySizes (Generic/ConfigurationBase.tt:80)
+static const int kArraySizes[] = {1, 31, 33, 127, 1027};
+
+// ITestSequencer (Generic/AlgorithmsTestData.tt:74-96)
+template <typename T> std::vector<T> ComputeSequence(T start, T step, int length) {
+  std::vector<T> s((size_t)length);
+  s[0] = start;
+  for (int i = 1; i < length; ++i) s[i] = (T)(s[i - 1] + step);
+  return s;
+}
+template <typename T> std::vector<T> ComputeInvertedSequence(T start, T step, int length) {
+  std::vector<T> s((size_t)length);
+  s[length - 1] = start;
+  for (int i = length - 2; i >= 0; --i) s[i] = (T)(s[i + 1] + step);
+  return s;
+}
+template <typename T> bool Verify(const std::vector<T>& got, const std::vector<T>& expected) {
+  return got.size() >= expected.size() &&
+         std::memcmp(got.data(), expected.data(), expected.size() * sizeof(T)) == 0;
+}
+
+// ---- RadixSortExtensionTests -------------------------------------------------
+template <typename T, typename TAsc, typename TDesc> void RadixTests(Accelerator& accl) {
+  for (int length : kArraySizes) {
+    auto stream = accl.CreateStream();
+    const auto seq = ComputeSequence<T>(0, 1, length);
+    const auto inv = ComputeInvertedSequence<T>(0, 1, length);
+    const Index1D tempSize = ComputeRadixSortTempStorageSize<T, TAsc>(accl, length);
+    auto tmp = accl.Allocate1D<int32_t>(tempSize);
+    {  // RadixWorstCaseAscending (:144-187)
+      auto input = accl.Allocate1D<T>(length);
+      input->CopyFromCPU(*stream, inv);
+      auto radixSort = CreateRadixSort<T, Stride1D::Dense, TAsc>(accl);
+      radixSort(*stream, input->View(), tmp->View());
+      stream->Synchronize();
+      CHECK(Verify(input->GetAsArray1D(), seq));
+    }
+    {  // RadixBestCaseAscending (:189-230)
+      auto input = accl.Allocate1D<T>(length);
+      input->CopyFromCPU(*stream, seq);
+      CreateRadixSort<T, Stride1D::Dense, TAsc>(accl)(*stream, input->View(), tmp->View());
+      stream->Synchronize();
+      CHECK(Verify(input->GetAsArray1D(), seq));
+    }
+    {  // RadixWorstCaseDescending
+      auto input = accl.Allocate1D<T>(length);
+      input->CopyFromCPU(*stream, seq);
+      CreateRadixSort<T, Stride1D::Dense, TDesc>(accl)(*stream, input->View(), tmp->View());
+      stream->Synchronize();
+      CHECK(Verify(input->GetAsArray1D(), inv));
+    }
+    {  // RadixProviderWorstCaseAscending (:232-317)
+      auto input = accl.Allocate1D<T>(length);
+      input->CopyFromCPU(*stream, inv);
+      auto provider = CreateRadixSortProvider<T, TAsc>(accl, length);
+      auto sortUsingProvider = provider->template CreateRadixSort<T, Stride1D::Dense, TAsc>();
+      sortUsingProvider(*stream, input->View());
+      stream->Synchronize();
+      CHECK(Verify(input->GetAsArray1D(), seq));
+    }
+    {  // RadixSortPairsAscending (:319-365): values == keys
+      auto keys = accl.Allocate1D<T>(length);
+      auto values = accl.Allocate1D<T>(length);
+      keys->CopyFromCPU(*stream, inv);
+      values->CopyFromCPU(*stream, inv);
+      auto sortPairs = CreateRadixSortPairs<T, Stride1D::Dense, T, Stride1D::Dense, TAsc>(accl);
+      auto tmpPairs = accl.Allocate1D<int32_t>(
+          ComputeRadixSortPairsTempStorageSize<T, T, TAsc>(accl, length));
+      sortPairs(*stream, keys->View(), values->View(), tmpPairs->View());
+      stream->Synchronize();
+      CHECK(Verify(keys->GetAsArray1D(), seq));
+      CHECK(Verify(values->GetAsArray1D(), seq));
+    }
+    // RadixConstCase (:370-432): start in {0, 1, -1}, step 0
+    for (int start : {0, 1, -1}) {
+      if (std::is_unsigned<T>::value && start < 0) continue;
+      const auto constant = ComputeSequence<T>((T)start, 0, length);
+      auto input = accl.Allocate1D<T>(length);
+      input->CopyFromCPU(*stream, constant);
+      CreateRadixSort<T, Stride1D::Dense, TAsc>(accl)(*stream, input->View(), tmp->View());
+      stream->Synchronize();
+      CHECK(Verify(input->GetAsArray1D(), constant));
+    }
+  }
+}
+
+static void RadixSortSequencerPairs(Accelerator& accl) {
+  // CreateRadixSortPairs with an index sequencer (RadixSortExtensions.cs:1017-1074)
+  const int n = 5003;
+  std::vector<uint32_t> keys((size_t)n);
+  for (int i = 0; i < n; ++i) keys[i] = (uint32_t)((i * 2654435761u) >> 24);  // many ties
+  std::vector<int32_t> order((size_t)n);
+  for (int i = 0; i < n; ++i) order[i] = i;
+  std::stable_sort(order.begin(), order.end(),
+                   [&](int a, int b) { return keys[a] < keys[b]; });
+  auto dKeys = accl.Allocate1D<uint32_t>(keys);
+  auto dValues = accl.Allocate1D<int32_t>(n);
+  auto tmp = accl.Allocate1D<int32_t>(
+      ComputeRadixSortPairsTempStorageSize<uint32_t, int32_t, RSO::AscendingUInt32>(accl, n));
+  auto sort = CreateRadixSortPairsWithSequencer<uint32_t, Stride1D::Dense, int32_t,
+                                                Stride1D::Dense, Sequencers::Int32Sequencer,
+                                                RSO::AscendingUInt32>(accl);
+  sort(accl.DefaultStream(), dKeys->View(), dValues->View(), Sequencers::Int32Sequencer(),
+       tmp->View());
+  accl.Synchronize();
+  CHECK(Verify(dValues->GetAsArray1D(), order));
+}
+
+static void RadixSortErrors(Accelerator& accl) {
+  auto sort = CreateRadixSort<int32_t, Stride1D::Dense, RSO::AscendingInt32>(accl);
+  auto data = accl.Allocate1D<int32_t>(64);
+  auto tmp = accl.Allocate1D<int32_t>(
+      ComputeRadixSortTempStorageSize<int32_t, RSO::AscendingInt32>(accl, 64));
+  auto& s = accl.DefaultStream();
+  EXPECT_THROW(sort(s, ArrayView<int32_t>(), tmp->View()), ArgumentNullException);
+  EXPECT_THROW(sort(s, data->View(), ArrayView<int32_t>()), ArgumentNullException);
+  EXPECT_THROW(sort(s, data->View(), tmp->View().SubView(0, 4)), ArgumentOutOfRangeException);
+  auto pairs = CreateRadixSortPairs<int32_t, Stride1D::Dense, int32_t, Stride1D::Dense,
+                                    RSO::AscendingInt32>(accl);
+  auto vals = accl.Allocate1D<int32_t>(32);
+  EXPECT_THROW(pairs(s, data->View(), vals->View(), tmp->View()), ArgumentOutOfRangeException);
+  EXPECT_THROW(RadixSortProvider(accl, 0), ArgumentOutOfRangeException);
+}
+
+// ---- ScanExtensionTests -------------------------------------------------------
+template <typename T, typename TOp>
+std::vector<T> CalcValues(const std::vector<T>& seq, ScanKind kind) {
+  // ScanExtensionTests.tt:286-305
+  std::vector<T> out(seq.size());
+  T acc = TOp::Identity();
+  for (size_t i = 0; i < seq.size(); ++i) {
+    T next;
+    if (TOp::Op == ILGPU_HIP_OP_ADD) next = (T)(acc + seq[i]);
+    else if (TOp::Op == ILGPU_HIP_OP_MAX) next = std::max(acc, seq[i]);
+    else next = std::min(acc, seq[i]);
+    out[i] = kind == ScanKind::Inclusive ? next : acc;
+    acc = next;
+  }
+  return out;
+}
+
+template <typename T, typename TOp> void ScanTests(Accelerator& accl, int maxLength) {
+  for (int length : kArraySizes) {
+    if (length > maxLength) continue;  // floats: :52
+    for (int variant = 0; variant < 3; ++variant) {
+      // ascending (0,1), constant (1,0), descending (length,-1) as inverted ascending
+      std::vector<T> seq = variant == 0   ? ComputeSequence<T>(0, 1, length)
+                           : variant == 1 ? ComputeSequence<T>(1, 0, length)
+                                          : ComputeInvertedSequence<T>(1, 1, length);
+      for (ScanKind kind : {ScanKind::Inclusive, ScanKind::Exclusive}) {
+        auto input = accl.Allocate1D<T>(seq);
+        auto output = accl.Allocate1D<T>(length);
+        auto scan = CreateScan<T, Stride1D::General, Stride1D::General, TOp>(accl, kind);
+        auto tmp = accl.Allocate1D<int32_t>((int64_t)ComputeScanTempStorageSize<T>(accl, length));
+        // the reference always goes through AsGeneral() views (:148-154)
+        ArrayView1D<T> in(input->View()), out(output->View());
+        scan(accl.DefaultStream(), in.AsGeneral(), out.AsGeneral(), tmp->View());
+        accl.Synchronize();
+        CHECK(Verify(output->GetAsArray1D(), CalcValues<T, TOp>(seq, kind)));
+      }
+    }
+  }
+}
+
+static void ScanErrors(Accelerator& accl) {
+  auto scan = CreateScan<int32_t, Stride1D::Dense, Stride1D::Dense, SRO::AddInt32>(
+      accl, ScanKind::Inclusive);
+  auto in = accl.Allocate1D<int32_t>(100);
+  auto out = accl.Allocate1D<int32_t>(100);
+  auto tmp = accl.Allocate1D<int32_t>((int64_t)ComputeScanTempStorageSize<int32_t>(accl, 100));
+  auto& s = accl.DefaultStream();
+  EXPECT_THROW(scan(s, ArrayView<int32_t>(), out->View(), tmp->View()), ArgumentNullException);
+  EXPECT_THROW(scan(s, in->View(), ArrayView<int32_t>(), tmp->View()), ArgumentNullException);
+  EXPECT_THROW(scan(s, in->View(), out->View().SubView(0, 50), tmp->View()),
+               ArgumentOutOfRangeException);
+  EXPECT_THROW(scan(s, in->View(), out->View(), ArrayView<int32_t>()), ArgumentNullException);
+  ArrayView1D<int32_t, Stride1D::General> strided(in->View(), 50, Stride1D::General{2});
+  auto gscan = CreateScan<int32_t, Stride1D::General, Stride1D::Dense, SRO::AddInt32>(
+      accl, ScanKind::Inclusive);
+  EXPECT_THROW(gscan(s, strided, out->View(), tmp->View()), NotSupportedException);
+  // provider variant
+  auto provider = CreateScanProvider<int32_t>(accl, 100);
+  auto buffered = provider->CreateScan<int32_t, Stride1D::Dense, Stride1D::Dense, SRO::AddInt32>(
+      ScanKind::Exclusive);
+  in->CopyFromCPU(std::vector<int32_t>(100, 2));
+  buffered(s, in->View(), out->View());
+  accl.Synchronize();
+  auto got = out->GetAsArray1D();
+  CHECK(got[0] == 0 && got[99] == 198);
+}
+
+// ---- ReductionExtensionTests ----------------------------------------------------
+template <typename T, typename TOp> void ReduceTests(Accelerator& accl, int maxLength) {
+  for (int length : kArraySizes) {
+    if (length > maxLength) continue;
+    for (int variant = 0; variant < 2; ++variant) {
+      const auto seq = variant == 0 ? ComputeSequence<T>(0, 1, length)
+                                    : ComputeSequence<T>(1, 0, length);
+      const T expected = CalcValues<T, TOp>(seq, ScanKind::Inclusive).back();  // left fold (:205-212)
+      auto input = accl.Allocate1D<T>(seq);
+      // value-returning overload with its cached output (:119-150)
+      const T got = Reduce<T, TOp>(accl, accl.DefaultStream(), input->View());
+      CHECK(got == expected);
+      // explicit output view (:152-196); output[0] is overwritten
+      auto output = accl.Allocate1D<T>(std::vector<T>{(T)77, (T)78});
+      Reduce<T, TOp>(accl, accl.DefaultStream(), input->View(), output->View());
+      accl.Synchronize();
+      auto o = output->GetAsArray1D();
+      CHECK(o[0] == expected && o[1] == (T)78);
+    }
+  }
+}
+
+static void ReduceErrors(Accelerator& accl) {
+  auto reduce = CreateReduction<float, Stride1D::Dense, SRO::AddFloat>(accl);
+  auto in = accl.Allocate1D<float>(10);
+  auto out = accl.Allocate1D<float>(1);
+  auto& s = accl.DefaultStream();
+  EXPECT_THROW(reduce(s, ArrayView<float>(), out->View()), ArgumentNullException);
+  EXPECT_THROW(reduce(s, in->View(), ArrayView<float>()), ArgumentNullException);
+}
+
+// ---- HistogramTests -----------------------------------------------------------
+template <typename T, typename TBin> void HistogramTests(Accelerator& accl) {
+  using Modulo = HistogramOperations::ModuloBinOperation;
+  for (int numBins : {64, 256}) {  // Histogram_CreateBin...(64|256, 1024) (:99-144)
+    const int length = 1024;
+    std::vector<T> input((size_t)length);
+    for (int i = 0; i < length; ++i) input[i] = (T)(i + 1);
+    std::vector<TBin> expected((size_t)numBins, 0);
+    for (T v : input) {
+      long bin;
+      if (std::is_floating_point<T>::value) bin = (long)std::fabs(std::fmod((double)v, (double)numBins));
+      else bin = std::labs((long)((long long)v % numBins));
+      expected[(size_t)bin] += 1;
+    }
+    auto dIn = accl.Allocate1D<T>(input);
+    auto hist = accl.Allocate1D<TBin>(numBins);
+    hist->MemSetToZero();
+    auto overflow = accl.Allocate1D<int32_t>(1);
+    overflow->MemSetToZero();
+    accl.Synchronize();
+    Histogram<T, Stride1D::Dense, Modulo, TBin>(accl, accl.DefaultStream(), dIn->View(),
+                                                hist->View(), overflow->View());
+    accl.Synchronize();
+    CHECK(Verify(hist->GetAsArray1D(), expected));
+    CHECK(overflow->GetAsArray1D()[0] == 0);
+  }
+  {  // HistogramOverflow_CreateBin... (:146-203)
+    const int length = 32;
+    std::vector<T> input((size_t)length);
+    for (int i = 0; i < length; ++i) input[i] = (T)(i + 1);
+    const TBin start = (TBin)(std::numeric_limits<TBin>::max() - (TBin)length - 1);
+    auto dIn = accl.Allocate1D<T>(input);
+    auto hist = accl.Allocate1D<TBin>(std::vector<TBin>{start});
+    auto overflow = accl.Allocate1D<int32_t>(1);
+    overflow->MemSetToZero();
+    using Unsigned = typename std::make_unsigned<TBin>::type;
+    Histogram<T, Stride1D::Dense, Modulo, TBin>(accl, accl.DefaultStream(), dIn->View(),
+                                                hist->View(), overflow->View());
+    accl.Synchronize();
+    CHECK(hist->GetAsArray1D()[0] == (TBin)((Unsigned)start + (Unsigned)length));
+    CHECK(overflow->GetAsArray1D()[0] == 0);
+    Histogram<T, Stride1D::Dense, Modulo, TBin>(accl, accl.DefaultStream(), dIn->View(),
+                                                hist->View(), overflow->View());
+    accl.Synchronize();
+    CHECK(hist->GetAsArray1D()[0] == (TBin)((Unsigned)start + (Unsigned)(2 * length)));
+    CHECK(overflow->GetAsArray1D()[0] == 1);
+  }
+}
+
+// ---- TempViewManagerTests (host only) ------------------------------------------
+template <typename T> void TempViewManagerTests() {
+  int32_t* fake = reinterpret_cast<int32_t*>(0x10000);  // never dereferenced
+  const int64_t rel = ((int64_t)sizeof(T) + 3) / 4;
+  {  // AlignedAllocation (TempViewManagerTests.cs:51-63)
+    TempViewManager m(ArrayView<int32_t>(fake, rel * 2), "buffer");
+    m.Allocate<T>(1);
+    m.Allocate<T>(1);
+    CHECK(m.NumInts() == rel * 2);
+  }
+  if (sizeof(T) > sizeof(int32_t)) {  // UnalignedAllocation (:65-84)
+    TempViewManager m(ArrayView<int32_t>(fake, rel + 1), "buffer");
+    m.Allocate<uint8_t>(1);
+    EXPECT_THROW(m.Allocate<T>(1), InvalidOperationException);
+  }
+  {
+    TempViewManager m(ArrayView<int32_t>(fake, rel), "buffer");
+    m.Allocate<T>(1);
+    EXPECT_THROW(m.Allocate<T>(1), ArgumentOutOfRangeException);
+  }
+  EXPECT_THROW(TempViewManager(ArrayView<int32_t>(), "temp"), ArgumentNullException);
+}
+
+int main(int argc, char** argv) {
+  const bool hostOnly = argc > 1 && std::string(argv[1]) == "--host";
+  RUN(TempViewManagerTests<int8_t>());
+  RUN(TempViewManagerTests<int32_t>());
+  RUN(TempViewManagerTests<int64_t>());
+  RUN(TempViewManagerTests<double>());
+  if (!hostOnly) {
+    Accelerator accl(0);
+    RUN((RadixTests<int32_t, RSO::AscendingInt32, RSO::DescendingInt32>(accl)));
+    RUN((RadixTests<int64_t, RSO::AscendingInt64, RSO::DescendingInt64>(accl)));
+    RUN((RadixTests<uint32_t, RSO::AscendingUInt32, RSO::DescendingUInt32>(accl)));
+    RUN((RadixTests<uint64_t, RSO::AscendingUInt64, RSO::DescendingUInt64>(accl)));
+    RUN((RadixTests<float, RSO::AscendingFloat, RSO::DescendingFloat>(accl)));
+    RUN((RadixTests<double, RSO::AscendingDouble, RSO::DescendingDouble>(accl)));
+    RUN(RadixSortSequencerPairs(accl));
+    RUN(RadixSortErrors(accl));
+    RUN((ScanTests<int32_t, SRO::AddInt32>(accl, 1027)));
+    RUN((ScanTests<int32_t, SRO::MaxInt32>(accl, 1027)));
+    RUN((ScanTests<int64_t, SRO::MinInt64>(accl, 1027)));
+    RUN((ScanTests<uint32_t, SRO::AddUInt32>(accl, 1027)));
+    RUN((ScanTests<uint64_t, SRO::MaxUInt64>(accl, 1027)));
+    RUN((ScanTests<float, SRO::AddFloat>(accl, 1000)));
+    RUN((ScanTests<double, SRO::MinDouble>(accl, 1000)));
+    RUN(ScanErrors(accl));
+    RUN((ReduceTests<int32_t, SRO::AddInt32>(accl, 1027)));
+    RUN((ReduceTests<int64_t, SRO::MaxInt64>(accl, 1027)));
+    RUN((ReduceTests<uint32_t, SRO::MinUInt32>(accl, 1027)));
+    RUN((ReduceTests<uint64_t, SRO::AddUInt64>(accl, 1027)));
+    RUN((ReduceTests<float, SRO::AddFloat>(accl, 1000)));
+    RUN((ReduceTests<double, SRO::MaxDouble>(accl, 1000)));
+    RUN(ReduceErrors(accl));
+    RUN((HistogramTests<int32_t, int32_t>(accl)));
+    RUN((HistogramTests<uint8_t, uint32_t>(accl)));
+    RUN((HistogramTests<int64_t, int64_t>(accl)));
+    RUN((HistogramTests<float, uint64_t>(accl)));
+    RUN((HistogramTests<int16_t, int32_t>(accl)));
+  }
+  std::printf("%d test groups, %d failed checks\n", g_run, g_failed);
+  return g_failed == 0 ? 0 : 1;
+}
