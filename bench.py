@@ -81,6 +81,17 @@ def kernel_stats(capi, name):
     return launches, (total_ms / launches if launches else 0.0)
 
 
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3
+# (FETCH_SIZE and WRITE_SIZE in separate runs of this script, each scaled by
+# what the same counter reads for a 1 GiB device copy: 2.00 and 1.00).  A
+# counter run cannot be nested inside this script, so the figure of the
+# committed profile is reported for the workload it was taken on.
+MEASURED_TRAFFIC_BYTES = {
+    # (kernel, log2 n): bytes per launch
+    ("onesweep_kernel<4,0>", 28): 2.98e9,
+}
+
+
 def roofline(achieved_gbs, traffic=None):
     return {"bound": "hbm", "achieved": round(achieved_gbs, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -194,7 +205,9 @@ def main():
                                "(SplitMix64 seed 0x123456789ABCDEF0)",
                    "n": n, "passes_executed": passes,
                    "algorithmic_bytes_per_key": 4 * (2 * passes + 1)},
-        "roofline": dict(roofline(pass_gbs), kernel="onesweep_kernel<4,0>",
+        "roofline": dict(roofline(pass_gbs, MEASURED_TRAFFIC_BYTES.get(
+                             ("onesweep_kernel<4,0>", args.log2n))),
+                         kernel="onesweep_kernel<4,0>",
                          bytes_per_launch=pass_bytes,
                          avg_launch_ms=round(pass_ms, 4),
                          launches=pass_launches),
