@@ -48,9 +48,6 @@ constexpr int kMaxPasses = 8;
 #ifndef ILGPU_HIP_SORT_ITEMS
 #define ILGPU_HIP_SORT_ITEMS 16
 #endif
-#ifndef ILGPU_HIP_SORT_WAVES_PER_EU
-#define ILGPU_HIP_SORT_WAVES_PER_EU 4
-#endif
 #ifndef ILGPU_HIP_SORT_LOOKBACK
 #define ILGPU_HIP_SORT_LOOKBACK 4
 #endif
@@ -231,8 +228,8 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 // Ranking.  A block's tile is cut into sub-tiles, one per half-wave (32
 // lanes); lane l of half-wave h holds items h*32*kItems + j*32 + l, j = 0 ..
 // kItems-1, so memory order inside a sub-tile is (row j, lane).  Every
-// (half-wave, digit) pair owns a peer-mask word and a running-count word in
-// LDS.  For row j every lane
+// (half-wave, digit) pair owns one 64-bit LDS slot: a peer-mask word and a
+// running-count word (read and rewritten together).  For row j every lane
 //   1. ORs its lane bit into the mask word of its digit (LDS atomic),
 //   2. reads mask and count back: the mask now names all lanes of the
 //      half-wave holding that digit in this row, the count is the number of
@@ -269,6 +266,20 @@ __device__ __forceinline__ void load_tile_keys(
   }
 }
 
+// Waves per SIMD the pass kernel is compiled for.  Keys-only sorts keep 16
+// keys and 8 registers of packed ranks per thread and fit 80 registers, so
+// three blocks share a CU; values add up to 16 x 16 bytes per thread.
+template <int VALUE_BYTES> constexpr int sort_waves_per_eu() {
+#ifdef ILGPU_HIP_SORT_WAVES_PER_EU
+  return ILGPU_HIP_SORT_WAVES_PER_EU;
+#else
+  return VALUE_BYTES == 0 ? 6 : 4;
+#endif
+}
+
+// Sorts one tile by the digit of `pass` and scatters it.  On return `key`
+// holds the keys of the block's next tile (ticket in `next_tile`), loaded
+// while this tile was written out.
 template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL>
 __device__ __forceinline__ void sort_tile(
     typename KeyOf<KEY_BYTES>::type (&key)[SortTile<KEY_BYTES>::kItems],
@@ -277,31 +288,32 @@ __device__ __forceinline__ void sort_tile(
     typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
     int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
     const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
-    unsigned char* s_stage, uint32_t* s_digit_start, uint32_t* s_global_off,
-    uint32_t* s_scan,
-    // Fetching the next tile: its ticket is drawn after this tile's look-back
-    // and its keys are loaded while this tile is staged and written out.
+    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan,
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int64_t n,
-    uint32_t* ticket, int num_tiles, int* s_next_tile, int& next_tile,
-    typename KeyOf<KEY_BYTES>::type (&next_key)[SortTile<KEY_BYTES>::kItems]) {
+    uint32_t* ticket, int num_tiles, int* s_next_tile, int& next_tile) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES>;
   constexpr int kItems = TileCfg::kItems;
   constexpr int kSubTiles = TileCfg::kSubTiles;
-  constexpr int kSlotWords = TileCfg::kSlotWords;
   constexpr bool kPairs = VALUE_BYTES > 0;
   constexpr int kValuesPerRound =
       kPairs ? TileCfg::kStageBytes / (VALUE_BYTES > 0 ? VALUE_BYTES : 1) : 1;
   constexpr int kRounds =
       kPairs ? (TileCfg::kTile + kValuesPerRound - 1) / kValuesPerRound : 0;
+  static_assert(kItems % 2 == 0 && TileCfg::kTile <= 65536,
+                "ranks and tile positions are packed two to a register");
 
-  uint32_t* s_mask = reinterpret_cast<uint32_t*>(s_stage);
-  uint32_t* s_count = s_mask + kSlotWords;
+  // Slot of (sub-tile, digit): {peer mask, running count}, one 64-bit word.
+  uint2* s_slot = reinterpret_cast<uint2*>(s_stage);
   K* s_keys = reinterpret_cast<K*>(s_stage);
   Val* s_vals = reinterpret_cast<Val*>(s_stage);
 
-  const int tid = threadIdx.x;
+  // The thread index is made opaque per tile (and again for the write-out):
+  // otherwise every per-item index derived from it is hoisted out of the
+  // tile loop and held in a register of its own, dozens of them.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
   const int lane = tid & (kWaveSize - 1);
   const int wave = tid / kWaveSize;
   const int sub = tid >> 5;                 // half-wave index in the block
@@ -314,6 +326,11 @@ __device__ __forceinline__ void sort_tile(
   auto digit = [&](K k) -> uint32_t {
     if constexpr (FLOAT_KEYS) return digit_of(k, xf, shift);
     else return (uint32_t)((K)(k ^ (K)xf.xor_mask) >> shift) & (kRadix - 1);
+  };
+  // Keys past the end of the input take digit 255; they come last in memory
+  // order, so they rank behind every real key and are dropped on write-out.
+  auto item_digit = [&](int j) -> uint32_t {
+    return (FULL || first_local + j * 32 < valid) ? digit(key[j]) : (uint32_t)(kRadix - 1);
   };
 
   Val val[kPairs ? kItems : 1];
@@ -332,30 +349,30 @@ __device__ __forceinline__ void sort_tile(
     }
   }
 
-  // Keys past the end of the input take digit 255; they come last in memory
-  // order, so they rank behind every real key and are dropped on write-out.
-  uint32_t* my_mask = s_mask + sub * kRadix;
-  uint32_t rank[kItems];
+  // Rank inside the sub-tile, later position inside the tile: 16 bits each.
+  uint2* my_slots = s_slot + sub * kRadix;
+  uint32_t packed[kItems / 2];
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
-    const int local = first_local + j * 32;
-    const uint32_t d = (FULL || local < valid) ? digit(key[j]) : (kRadix - 1);
-    uint32_t* mask_word = my_mask + d;
-    uint32_t* count_word = mask_word + kSlotWords;
-    __hip_atomic_fetch_or(mask_word, lane_bit, __ATOMIC_RELAXED,
+    uint2* slot = my_slots + item_digit(j);
+    __hip_atomic_fetch_or(&slot->x, lane_bit, __ATOMIC_RELAXED,
                           __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint32_t peers = __hip_atomic_load(mask_word, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint32_t before = __hip_atomic_load(count_word, __ATOMIC_RELAXED,
-                                              __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint64_t both = __hip_atomic_load(reinterpret_cast<uint64_t*>(slot),
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t peers = (uint32_t)both;
+    const uint32_t before = (uint32_t)(both >> 32);
     const uint32_t below = (uint32_t)__popc(peers & lower_lanes);
-    if (below == 0) {
-      __hip_atomic_store(count_word, before + (uint32_t)__popc(peers),
+    if (below == 0)  // new count, mask cleared for the next row
+      __hip_atomic_store(reinterpret_cast<uint64_t*>(slot),
+                         (uint64_t)(before + (uint32_t)__popc(peers)) << 32,
                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      __hip_atomic_store(mask_word, 0u, __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-    rank[j] = before + below;
+    const uint32_t rank = before + below;
+    if (j % 2 == 0) packed[j / 2] = rank;
+    else packed[j / 2] |= rank << 16;
+    // Rows chain through LDS anyway.  Pin the packed rank here: left alone,
+    // the compiler sinks the rank arithmetic of all rows to where the ranks
+    // are used and keeps two live registers per key until then.
+    asm volatile("" : "+v"(packed[j / 2]));
   }
   __syncthreads();
 
@@ -364,11 +381,7 @@ __device__ __forceinline__ void sort_tile(
   uint32_t* tile_status = status + (int64_t)tile * kRadix;
   if (tid < kRadix) {
 #pragma unroll
-    for (int s = 0; s < kSubTiles; ++s) {
-      const uint32_t t = s_count[s * kRadix + tid];
-      s_count[s * kRadix + tid] = count;
-      count += t;
-    }
+    for (int s = 0; s < kSubTiles; ++s) count += s_slot[s * kRadix + tid].y;
     __hip_atomic_store(&tile_status[tid],
                        (tile == 0 ? kStatusPrefix : kStatusAggregate) | count,
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -384,7 +397,16 @@ __device__ __forceinline__ void sort_tile(
   if (tid < kRadix) {
     uint32_t digit_start = inc - count;
     for (int w = 0; w < wave; ++w) digit_start += s_scan[w];
-    s_digit_start[tid] = digit_start;
+    // Tile-local position of the first key of every (sub-tile, digit) run.
+    {
+      uint32_t run = digit_start;
+#pragma unroll
+      for (int s = 0; s < kSubTiles; ++s) {
+        const uint32_t t = s_slot[s * kRadix + tid].y;
+        s_slot[s * kRadix + tid].y = run;
+        run += t;
+      }
+    }
 
     // Keys with this digit in earlier tiles: walk back over the status words,
     // kLookback tiles per step.  The loads of a step are unconditional (index
@@ -423,33 +445,37 @@ __device__ __forceinline__ void sort_tile(
   }
   __syncthreads();
   next_tile = *s_next_tile;
+
+  // Tile-local position of every key; afterwards the slots are dead and the
+  // same LDS bytes stage the keys in digit order.
+#pragma unroll
+  for (int j = 0; j < kItems; j += 2) {
+    const uint32_t p0 = my_slots[item_digit(j)].y + (packed[j / 2] & 0xFFFFu);
+    const uint32_t p1 = my_slots[item_digit(j + 1)].y + (packed[j / 2] >> 16);
+    packed[j / 2] = p0 | (p1 << 16);
+    if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kItems; ++j)
+    s_keys[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = key[j];
+  __syncthreads();
+
+  // The key registers are free: fetch the next tile during the write-out.
   {
     const int64_t next_base = (int64_t)next_tile * TileCfg::kTile;
     const int64_t remaining = n - next_base;
     if (next_tile < num_tiles && remaining >= TileCfg::kTile)
-      load_tile_keys<KEY_BYTES, true>(src_keys, next_base, TileCfg::kTile, first_local, next_key);
+      load_tile_keys<KEY_BYTES, true>(src_keys, next_base, TileCfg::kTile, first_local, key);
     else
       load_tile_keys<KEY_BYTES, false>(
           src_keys, next_base,
           next_tile < num_tiles && remaining > 0 ? (int)remaining : 0,
-          first_local, next_key);
+          first_local, key);
   }
-
-  // Tile-local position of every key; afterwards the mask/count words are
-  // dead and the same LDS bytes stage the keys in digit order.
-  uint32_t pos[kItems];
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    const int local = first_local + j * 32;
-    const uint32_t d = (FULL || local < valid) ? digit(key[j]) : (kRadix - 1);
-    pos[j] = s_count[sub * kRadix + d] + s_digit_start[d] + rank[j];
-  }
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) s_keys[pos[j]] = key[j];
-  __syncthreads();
 
   uint32_t gpos[kPairs ? kItems : 1];
+  asm volatile("" : "+v"(tid));
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
     const int i = j * kSortBlock + tid;
@@ -459,6 +485,7 @@ __device__ __forceinline__ void sort_tile(
       dst_keys[g] = k;
       if constexpr (kPairs) gpos[j] = g;
     }
+    if (j % 4 == 3) __builtin_amdgcn_sched_barrier(0);
   }
 
   if constexpr (kPairs) {
@@ -467,8 +494,10 @@ __device__ __forceinline__ void sort_tile(
       const uint32_t lo = (uint32_t)r * kValuesPerRound;
       __syncthreads();  // the stage buffer is free again
 #pragma unroll
-      for (int j = 0; j < kItems; ++j)
-        if (pos[j] - lo < (uint32_t)kValuesPerRound) s_vals[pos[j] - lo] = val[j];
+      for (int j = 0; j < kItems; ++j) {
+        const uint32_t pos = j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16;
+        if (pos - lo < (uint32_t)kValuesPerRound) s_vals[pos - lo] = val[j];
+      }
       __syncthreads();
 #pragma unroll
       for (int j = 0; j < kItems; ++j) {
@@ -481,7 +510,7 @@ __device__ __forceinline__ void sort_tile(
 }
 
 template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS>
-__global__ __launch_bounds__(kSortBlock, ILGPU_HIP_SORT_WAVES_PER_EU)
+__global__ __launch_bounds__(kSortBlock, sort_waves_per_eu<VALUE_BYTES>())
 void onesweep_kernel(
     typename KeyOf<KEY_BYTES>::type* keys_a,
     typename KeyOf<KEY_BYTES>::type* keys_b,
@@ -497,7 +526,6 @@ void onesweep_kernel(
   constexpr int kItems = TileCfg::kItems;
 
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[TileCfg::kStageBytes];
-  __shared__ uint32_t s_digit_start[kRadix];
   __shared__ uint32_t s_global_off[kRadix];
   __shared__ uint32_t s_scan[kRadix / kWaveSize];
   __shared__ int s_tile[2];
@@ -537,20 +565,17 @@ void onesweep_kernel(
     const int64_t tile_base = (int64_t)tile * kTile;
     const int valid = valid_keys(tile);
     int next = num_tiles;
-    K next_key[kItems];
     if (valid == kTile) {
       sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, true>(
           key, dst_keys, src_vals, dst_vals, tile_base, kTile, tile, pass, xf,
-          excl, status, make_index, s_stage, s_digit_start, s_global_off, s_scan,
-          src_keys, n, ticket, num_tiles, &s_tile[1], next, next_key);
+          excl, status, make_index, s_stage, s_global_off, s_scan,
+          src_keys, n, ticket, num_tiles, &s_tile[1], next);
     } else {
       sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false>(
           key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
-          excl, status, make_index, s_stage, s_digit_start, s_global_off, s_scan,
-          src_keys, n, ticket, num_tiles, &s_tile[1], next, next_key);
+          excl, status, make_index, s_stage, s_global_off, s_scan,
+          src_keys, n, ticket, num_tiles, &s_tile[1], next);
     }
-#pragma unroll
-    for (int j = 0; j < kItems; ++j) key[j] = next_key[j];
     tile = next;
     __syncthreads();  // LDS is reused by the next tile
   }
