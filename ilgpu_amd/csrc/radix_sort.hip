@@ -46,7 +46,10 @@ constexpr int kMaxPasses = 8;
 #define ILGPU_HIP_SORT_BLOCK 512
 #endif
 #ifndef ILGPU_HIP_SORT_ITEMS
-#define ILGPU_HIP_SORT_ITEMS 16
+#define ILGPU_HIP_SORT_ITEMS 28
+#endif
+#ifndef ILGPU_HIP_SORT_PAIR_ITEMS
+#define ILGPU_HIP_SORT_PAIR_ITEMS 16
 #endif
 #ifndef ILGPU_HIP_SORT_LOOKBACK
 #define ILGPU_HIP_SORT_LOOKBACK 4
@@ -72,12 +75,17 @@ template <> struct ValueOf<4> { using type = uint32_t; };
 template <> struct ValueOf<8> { using type = uint64_t; };
 template <> struct ValueOf<16> { using type = Bytes16; };
 
-template <int KEY_BYTES> constexpr int items_per_thread() {
-  // 8-byte keys take two registers each: half the items, same bytes per tile.
-  return KEY_BYTES == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_ITEMS;
+// Keys per thread and tile.  Keys-only sorts take long tiles: the runs they
+// scatter are longer (fewer partial cache lines) and there are fewer tiles
+// to chain.  Values live in registers next to the keys, so pairs take the
+// short tile.  8-byte keys take two registers each: half the items, same
+// bytes per tile.
+constexpr int items_per_thread(int key_bytes, int value_bytes) {
+  const int items = value_bytes == 0 ? ILGPU_HIP_SORT_ITEMS : ILGPU_HIP_SORT_PAIR_ITEMS;
+  return key_bytes == 8 ? items / 2 : items;
 }
-template <int KEY_BYTES> constexpr int tile_keys() {
-  return kSortBlock * items_per_thread<KEY_BYTES>();
+constexpr int tile_keys(int key_bytes, int value_bytes) {
+  return kSortBlock * items_per_thread(key_bytes, value_bytes);
 }
 
 // How raw key bits map to unsigned bits that sort in the requested order.
@@ -241,48 +249,44 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 // through the two words without barriers, and equal digits keep memory
 // order: the pass is stable.  No ballots: the cost per key is a handful of
 // LDS operations and about ten VALU operations whatever the key distribution.
-template <int KEY_BYTES> struct SortTile {
+template <int KEY_BYTES, int VALUE_BYTES> struct SortTile {
   static constexpr int kSubTiles = kSortBlock / 32;
   static constexpr int kSlotWords = kSubTiles * kRadix;      // per array
   static constexpr int kSlotBytes = 2 * kSlotWords * 4;      // masks + counts
-  static constexpr int kItems = items_per_thread<KEY_BYTES>();
-  static constexpr int kTile = tile_keys<KEY_BYTES>();
+  static constexpr int kItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
+  static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES);
   static constexpr int kSubTileKeys = 32 * kItems;
   static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
   static constexpr int kStageBytes =
       kSlotBytes > kKeyStageBytes ? kSlotBytes : kKeyStageBytes;
 };
 
-template <int KEY_BYTES, bool FULL>
+template <int KEY_BYTES, int ITEMS, bool FULL>
 __device__ __forceinline__ void load_tile_keys(
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src, int64_t tile_base,
     int valid, int first_local,
-    typename KeyOf<KEY_BYTES>::type (&key)[SortTile<KEY_BYTES>::kItems]) {
+    typename KeyOf<KEY_BYTES>::type (&key)[ITEMS]) {
 #pragma unroll
-  for (int j = 0; j < SortTile<KEY_BYTES>::kItems; ++j) {
+  for (int j = 0; j < ITEMS; ++j) {
     const int local = first_local + j * 32;
     if (FULL || local < valid) key[j] = src[tile_base + local];
     else key[j] = 0;
   }
 }
 
-// Waves per SIMD the pass kernel is compiled for.  Keys-only sorts keep 16
-// keys and 8 registers of packed ranks per thread and fit 80 registers, so
-// three blocks share a CU; values add up to 16 x 16 bytes per thread.
-template <int VALUE_BYTES> constexpr int sort_waves_per_eu() {
-#ifdef ILGPU_HIP_SORT_WAVES_PER_EU
-  return ILGPU_HIP_SORT_WAVES_PER_EU;
-#else
-  return VALUE_BYTES == 0 ? 6 : 4;
+// Waves per SIMD the pass kernel is compiled for: two blocks of eight waves
+// per CU.  That bounds a thread at 128 registers (28 keys, 14 registers of
+// packed ranks and the values of a pair fit) and a block at 80 KiB of LDS.
+#ifndef ILGPU_HIP_SORT_WAVES_PER_EU
+#define ILGPU_HIP_SORT_WAVES_PER_EU 4
 #endif
-}
 
 // Sorts one tile by the digit of `pass` and scatters it.  On return `key`
 // holds the keys of the block's next tile (ticket in `next_tile`), loaded
 // while this tile was written out.
 template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL>
 __device__ __forceinline__ void sort_tile(
-    typename KeyOf<KEY_BYTES>::type (&key)[SortTile<KEY_BYTES>::kItems],
+    typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
     typename KeyOf<KEY_BYTES>::type* __restrict__ dst_keys,
     const typename ValueOf<VALUE_BYTES>::type* __restrict__ src_vals,
     typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
@@ -293,7 +297,7 @@ __device__ __forceinline__ void sort_tile(
     uint32_t* ticket, int num_tiles, int* s_next_tile, int& next_tile) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES>;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
   constexpr int kItems = TileCfg::kItems;
   constexpr int kSubTiles = TileCfg::kSubTiles;
   constexpr bool kPairs = VALUE_BYTES > 0;
@@ -466,9 +470,9 @@ __device__ __forceinline__ void sort_tile(
     const int64_t next_base = (int64_t)next_tile * TileCfg::kTile;
     const int64_t remaining = n - next_base;
     if (next_tile < num_tiles && remaining >= TileCfg::kTile)
-      load_tile_keys<KEY_BYTES, true>(src_keys, next_base, TileCfg::kTile, first_local, key);
+      load_tile_keys<KEY_BYTES, kItems, true>(src_keys, next_base, TileCfg::kTile, first_local, key);
     else
-      load_tile_keys<KEY_BYTES, false>(
+      load_tile_keys<KEY_BYTES, kItems, false>(
           src_keys, next_base,
           next_tile < num_tiles && remaining > 0 ? (int)remaining : 0,
           first_local, key);
@@ -510,7 +514,7 @@ __device__ __forceinline__ void sort_tile(
 }
 
 template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS>
-__global__ __launch_bounds__(kSortBlock, sort_waves_per_eu<VALUE_BYTES>())
+__global__ __launch_bounds__(kSortBlock, ILGPU_HIP_SORT_WAVES_PER_EU)
 void onesweep_kernel(
     typename KeyOf<KEY_BYTES>::type* keys_a,
     typename KeyOf<KEY_BYTES>::type* keys_b,
@@ -521,7 +525,7 @@ void onesweep_kernel(
     int values_from_index) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES>;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
   constexpr int kTile = TileCfg::kTile;
   constexpr int kItems = TileCfg::kItems;
 
@@ -552,8 +556,8 @@ void onesweep_kernel(
   K key[kItems];
   if (tile < num_tiles) {
     const int valid = valid_keys(tile);
-    if (valid == kTile) load_tile_keys<KEY_BYTES, true>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
-    else load_tile_keys<KEY_BYTES, false>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
+    if (valid == kTile) load_tile_keys<KEY_BYTES, kItems, true>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
+    else load_tile_keys<KEY_BYTES, kItems, false>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
   }
   while (tile < num_tiles) {
     {  // clear the mask and count words
@@ -616,7 +620,7 @@ struct TempLayout {
 
 TempLayout make_layout(int64_t n, int key_bytes, int value_bytes) {
   TempLayout L;
-  const int64_t tile = key_bytes == 8 ? tile_keys<8>() : tile_keys<4>();
+  const int64_t tile = tile_keys(key_bytes, value_bytes);
   L.tiles = div_up(n, tile);
   int64_t off = 0;
   L.alt_keys = off; off += align_up(n * key_bytes, 256);
