@@ -55,6 +55,10 @@ constexpr int kMaxPasses = 8;
 #define ILGPU_HIP_SORT_LOOKBACK 4
 #endif
 constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;
+// Lanes that rank together (a sub-tile row): a quarter of a wave, so that a
+// peer mask and a running count share one 32-bit LDS word.
+constexpr int kSubLanes = 16;
+constexpr uint32_t kSubLaneMask = (1u << kSubLanes) - 1u;
 constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
 constexpr int kHistBlock = 512;
 constexpr uint32_t kStatusAggregate = 1u << 30;
@@ -233,29 +237,30 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 }
 
 // ---- onesweep pass ---------------------------------------------------------
-// Ranking.  A block's tile is cut into sub-tiles, one per half-wave (32
-// lanes); lane l of half-wave h holds items h*32*kItems + j*32 + l, j = 0 ..
-// kItems-1, so memory order inside a sub-tile is (row j, lane).  Every
-// (half-wave, digit) pair owns one 64-bit LDS slot: a peer-mask word and a
-// running-count word (read and rewritten together).  For row j every lane
-//   1. ORs its lane bit into the mask word of its digit (LDS atomic),
-//   2. reads mask and count back: the mask now names all lanes of the
-//      half-wave holding that digit in this row, the count is the number of
-//      keys with the digit in earlier rows,
+// Ranking.  A block's tile is cut into sub-tiles, one per quarter-wave (16
+// lanes); lane l of quarter-wave q holds items q*16*kItems + j*16 + l, j = 0
+// .. kItems-1, so memory order inside a sub-tile is (row j, lane).  Every
+// (quarter-wave, digit) pair owns one 32-bit LDS slot: a 16-bit peer mask
+// under a 16-bit running count.  For row j every lane
+//   1. ORs its lane bit into the slot of its digit (LDS atomic),
+//   2. reads the slot back: the mask now names all lanes of the quarter-wave
+//      holding that digit in this row, the count is the number of keys with
+//      the digit in earlier rows,
 //   3. ranks itself: count + number of peers in lower lanes,
-//   4. and the lowest peer stores count + number of peers and clears the mask
-//      for the next row.
+//   4. and the lowest peer stores count + number of peers with the mask
+//      cleared for the next row.
 // LDS instructions of one wave execute in issue order, so the rows chain
-// through the two words without barriers, and equal digits keep memory
-// order: the pass is stable.  No ballots: the cost per key is a handful of
-// LDS operations and about ten VALU operations whatever the key distribution.
+// through the slot without barriers, and equal digits keep memory order: the
+// pass is stable.  No ballots: the cost per key is three LDS operations on
+// 32-bit words (the cheapest the LDS offers for scattered addresses) and
+// about ten VALU operations whatever the key distribution.
 template <int KEY_BYTES, int VALUE_BYTES> struct SortTile {
-  static constexpr int kSubTiles = kSortBlock / 32;
-  static constexpr int kSlotWords = kSubTiles * kRadix;      // per array
-  static constexpr int kSlotBytes = 2 * kSlotWords * 4;      // masks + counts
+  static constexpr int kSubTiles = kSortBlock / kSubLanes;
+  static constexpr int kSlotWords = kSubTiles * kRadix;
+  static constexpr int kSlotBytes = kSlotWords * 4;
   static constexpr int kItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
   static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES);
-  static constexpr int kSubTileKeys = 32 * kItems;
+  static constexpr int kSubTileKeys = kSubLanes * kItems;
   static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
   static constexpr int kStageBytes =
       kSlotBytes > kKeyStageBytes ? kSlotBytes : kKeyStageBytes;
@@ -268,7 +273,7 @@ __device__ __forceinline__ void load_tile_keys(
     typename KeyOf<KEY_BYTES>::type (&key)[ITEMS]) {
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
-    const int local = first_local + j * 32;
+    const int local = first_local + j * kSubLanes;
     if (FULL || local < valid) key[j] = src[tile_base + local];
     else key[j] = 0;
   }
@@ -307,9 +312,10 @@ __device__ __forceinline__ void sort_tile(
       kPairs ? (TileCfg::kTile + kValuesPerRound - 1) / kValuesPerRound : 0;
   static_assert(kItems % 2 == 0 && TileCfg::kTile <= 65536,
                 "ranks and tile positions are packed two to a register");
+  static_assert(kItems * kSubLanes < 65536, "a sub-tile's digit count fits 16 bits");
 
-  // Slot of (sub-tile, digit): {peer mask, running count}, one 64-bit word.
-  uint2* s_slot = reinterpret_cast<uint2*>(s_stage);
+  // Slot of (sub-tile, digit): running count << 16 | peer mask.
+  uint32_t* s_slot = reinterpret_cast<uint32_t*>(s_stage);
   K* s_keys = reinterpret_cast<K*>(s_stage);
   Val* s_vals = reinterpret_cast<Val*>(s_stage);
 
@@ -320,8 +326,8 @@ __device__ __forceinline__ void sort_tile(
   asm volatile("" : "+v"(tid));
   const int lane = tid & (kWaveSize - 1);
   const int wave = tid / kWaveSize;
-  const int sub = tid >> 5;                 // half-wave index in the block
-  const int sub_lane = tid & 31;
+  const int sub = tid / kSubLanes;          // quarter-wave index in the block
+  const int sub_lane = tid % kSubLanes;
   const uint32_t lane_bit = 1u << sub_lane;
   const uint32_t lower_lanes = lane_bit - 1u;
   const int first_local = sub * TileCfg::kSubTileKeys + sub_lane;
@@ -334,14 +340,15 @@ __device__ __forceinline__ void sort_tile(
   // Keys past the end of the input take digit 255; they come last in memory
   // order, so they rank behind every real key and are dropped on write-out.
   auto item_digit = [&](int j) -> uint32_t {
-    return (FULL || first_local + j * 32 < valid) ? digit(key[j]) : (uint32_t)(kRadix - 1);
+    return (FULL || first_local + j * kSubLanes < valid) ? digit(key[j])
+                                                          : (uint32_t)(kRadix - 1);
   };
 
   Val val[kPairs ? kItems : 1];
   if constexpr (kPairs) {
 #pragma unroll
     for (int j = 0; j < kItems; ++j) {
-      const int local = first_local + j * 32;
+      const int local = first_local + j * kSubLanes;
       if (FULL || local < valid) {
         if (make_index) {
           if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)(tile_base + local);
@@ -354,21 +361,19 @@ __device__ __forceinline__ void sort_tile(
   }
 
   // Rank inside the sub-tile, later position inside the tile: 16 bits each.
-  uint2* my_slots = s_slot + sub * kRadix;
+  uint32_t* my_slots = s_slot + sub * kRadix;
   uint32_t packed[kItems / 2];
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
-    uint2* slot = my_slots + item_digit(j);
-    __hip_atomic_fetch_or(&slot->x, lane_bit, __ATOMIC_RELAXED,
-                          __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint64_t both = __hip_atomic_load(reinterpret_cast<uint64_t*>(slot),
-                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint32_t peers = (uint32_t)both;
-    const uint32_t before = (uint32_t)(both >> 32);
+    uint32_t* slot = my_slots + item_digit(j);
+    __hip_atomic_fetch_or(slot, lane_bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t both = __hip_atomic_load(slot, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t peers = both & kSubLaneMask;
+    const uint32_t before = both >> 16;
     const uint32_t below = (uint32_t)__popc(peers & lower_lanes);
     if (below == 0)  // new count, mask cleared for the next row
-      __hip_atomic_store(reinterpret_cast<uint64_t*>(slot),
-                         (uint64_t)(before + (uint32_t)__popc(peers)) << 32,
+      __hip_atomic_store(slot, (before + (uint32_t)__popc(peers)) << 16,
                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     const uint32_t rank = before + below;
     if (j % 2 == 0) packed[j / 2] = rank;
@@ -385,7 +390,7 @@ __device__ __forceinline__ void sort_tile(
   uint32_t* tile_status = status + (int64_t)tile * kRadix;
   if (tid < kRadix) {
 #pragma unroll
-    for (int s = 0; s < kSubTiles; ++s) count += s_slot[s * kRadix + tid].y;
+    for (int s = 0; s < kSubTiles; ++s) count += s_slot[s * kRadix + tid] >> 16;
     __hip_atomic_store(&tile_status[tid],
                        (tile == 0 ? kStatusPrefix : kStatusAggregate) | count,
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -406,8 +411,8 @@ __device__ __forceinline__ void sort_tile(
       uint32_t run = digit_start;
 #pragma unroll
       for (int s = 0; s < kSubTiles; ++s) {
-        const uint32_t t = s_slot[s * kRadix + tid].y;
-        s_slot[s * kRadix + tid].y = run;
+        const uint32_t t = s_slot[s * kRadix + tid] >> 16;
+        s_slot[s * kRadix + tid] = run;
         run += t;
       }
     }
@@ -454,8 +459,8 @@ __device__ __forceinline__ void sort_tile(
   // same LDS bytes stage the keys in digit order.
 #pragma unroll
   for (int j = 0; j < kItems; j += 2) {
-    const uint32_t p0 = my_slots[item_digit(j)].y + (packed[j / 2] & 0xFFFFu);
-    const uint32_t p1 = my_slots[item_digit(j + 1)].y + (packed[j / 2] >> 16);
+    const uint32_t p0 = my_slots[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
+    const uint32_t p1 = my_slots[item_digit(j + 1)] + (packed[j / 2] >> 16);
     packed[j / 2] = p0 | (p1 << 16);
     if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
   }
@@ -543,7 +548,7 @@ void onesweep_kernel(
   const bool make_index = VALUE_BYTES > 0 && values_from_index &&
                           plan->first_executed == (uint32_t)pass;
   const int tid = threadIdx.x;
-  const int first_local = (tid >> 5) * TileCfg::kSubTileKeys + (tid & 31);
+  const int first_local = (tid / kSubLanes) * TileCfg::kSubTileKeys + tid % kSubLanes;
 
   auto valid_keys = [&](int t) -> int {
     const int64_t remaining = n - (int64_t)t * kTile;
