@@ -40,6 +40,7 @@ EXPORTS = [
     "ilgpu_hip_version", "ilgpu_hip_status_string",
     "ilgpu_hip_last_runtime_error", "ilgpu_hip_profile_enable",
     "ilgpu_hip_profile_query", "ilgpu_hip_radix_sort_temp_bytes",
+    "ilgpu_hip_radix_sort_temp_bytes_strided",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
@@ -117,6 +118,8 @@ def lib() -> ctypes.CDLL:
             ctypes.c_char_p, p64, ctypes.POINTER(ctypes.c_double)]
         L.ilgpu_hip_profile_query.restype = i32
         L.ilgpu_hip_radix_sort_temp_bytes.argtypes = [i64, i32, i32, p64]
+        L.ilgpu_hip_radix_sort_temp_bytes_strided.argtypes = [
+            i64, i32, i32, i64, i64, p64]
         L.ilgpu_hip_radix_sort_keys.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64]
         L.ilgpu_hip_radix_sort_pairs.argtypes = [
             vp, vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, i64]
@@ -169,6 +172,7 @@ class DeviceArray:
         nbytes = self.length * self.dtype.itemsize
         self.bytes = _bytes if _bytes is not None else torch.empty(
             max(nbytes, 1), dtype=torch.uint8, device="cuda:0")
+        self.stride = 1  # element stride (Stride1D.General when above one)
 
     @classmethod
     def from_numpy(cls, a: np.ndarray) -> "DeviceArray":
@@ -205,6 +209,15 @@ class DeviceArray:
     def clone(self) -> "DeviceArray":
         return DeviceArray(self.length, self.dtype, _bytes=self.bytes.clone())
 
+    def strided(self, stride: int) -> "DeviceArray":
+        """Every ``stride``-th element of this array as a view on the same
+        memory (``AsGeneral(new Stride1D.General(stride))``): element i of the
+        view is element ``i * stride`` of the array."""
+        view = DeviceArray((self.length + stride - 1) // stride, self.dtype,
+                           _bytes=self.bytes)
+        view.stride = int(stride)
+        return view
+
     def subview(self, offset: int, length: int) -> "DeviceArray":
         """Elements [offset, offset+length) as a view on the same memory."""
         s = self.dtype.itemsize
@@ -231,16 +244,23 @@ def _query(fn, *args) -> int:
 
 
 # ---- thin wrappers, one per entry point -------------------------------------
-def radix_sort_temp_bytes(n: int, key_dtype, value_bytes: int = 0) -> int:
+def radix_sort_temp_bytes(n: int, key_dtype, value_bytes: int = 0,
+                          key_stride: int = 1, value_stride: int = 1) -> int:
+    if key_stride != 1 or value_stride != 1:
+        return _query(lib().ilgpu_hip_radix_sort_temp_bytes_strided, n,
+                      type_code(key_dtype), value_bytes, key_stride,
+                      value_stride)
     return _query(lib().ilgpu_hip_radix_sort_temp_bytes, n,
                   type_code(key_dtype), value_bytes)
 
 
 def radix_sort_keys(keys: DeviceArray, temp: Optional[DeviceArray] = None, *,
                     descending: bool = False, float_total_order: bool = False,
-                    stream=None, stride: int = 1) -> None:
+                    stream=None, stride: Optional[int] = None) -> None:
+    stride = keys.stride if stride is None else stride
     if temp is None:
-        temp = temp_buffer(radix_sort_temp_bytes(keys.length, keys.dtype))
+        temp = temp_buffer(radix_sort_temp_bytes(keys.length, keys.dtype, 0,
+                                                 stride))
     flags = (SORT_DESCENDING if descending else 0) | (
         SORT_FLOAT_TOTAL_ORDER if float_total_order else 0)
     check(lib().ilgpu_hip_radix_sort_keys(
@@ -253,15 +273,17 @@ def radix_sort_pairs(keys: DeviceArray, values: DeviceArray,
                      descending: bool = False, float_total_order: bool = False,
                      values_from_index: bool = False, stream=None) -> None:
     if temp is None:
-        temp = temp_buffer(radix_sort_temp_bytes(keys.length, keys.dtype,
-                                                 values.dtype.itemsize))
+        temp = temp_buffer(radix_sort_temp_bytes(
+            keys.length, keys.dtype, values.dtype.itemsize, keys.stride,
+            values.stride))
     flags = (SORT_DESCENDING if descending else 0) | (
         SORT_FLOAT_TOTAL_ORDER if float_total_order else 0)
     if values.length != keys.length:
         # RadixSortExtensions.cs:1053-1054
         raise ArgumentOutOfRangeError(ERROR_OUT_OF_RANGE, "values")
     check(lib().ilgpu_hip_radix_sort_pairs(
-        _stream_ptr(stream), keys.ptr, 1, values.ptr, 1, keys.length,
+        _stream_ptr(stream), keys.ptr, keys.stride, values.ptr, values.stride,
+        keys.length,
         keys.type_code, values.dtype.itemsize, flags,
         VALUES_FROM_INDEX if values_from_index else VALUES_FROM_VIEW,
         temp.ptr, temp.nbytes))
@@ -276,8 +298,8 @@ def scan(inp: DeviceArray, out: DeviceArray, temp: Optional[DeviceArray] = None,
     if temp is None:
         temp = temp_buffer(scan_temp_bytes(max(inp.length, 1), inp.dtype))
     check(lib().ilgpu_hip_scan(
-        _stream_ptr(stream), inp.ptr, inp.length, 1, out.ptr, out.length, 1,
-        inp.type_code, op, kind, temp.ptr, temp.nbytes))
+        _stream_ptr(stream), inp.ptr, inp.length, inp.stride, out.ptr,
+        out.length, out.stride, inp.type_code, op, kind, temp.ptr, temp.nbytes))
 
 
 def reduce_temp_bytes(n: int, dtype) -> int:
@@ -290,14 +312,15 @@ def reduce(inp: DeviceArray, out: DeviceArray,
     if temp is None:
         temp = temp_buffer(reduce_temp_bytes(max(inp.length, 1), inp.dtype))
     check(lib().ilgpu_hip_reduce(
-        _stream_ptr(stream), inp.ptr, inp.length, 1, inp.type_code, op,
-        out.ptr, out.length, temp.ptr, temp.nbytes))
+        _stream_ptr(stream), inp.ptr, inp.length, inp.stride, inp.type_code,
+        op, out.ptr, out.length, temp.ptr, temp.nbytes))
 
 
 def histogram(inp: DeviceArray, bins: DeviceArray,
               overflow: Optional[DeviceArray] = None, *,
               locator: int = LOCATOR_IDENTITY, stream=None) -> None:
     check(lib().ilgpu_hip_histogram(
-        _stream_ptr(stream), inp.ptr, inp.length, 1, inp.type_code, bins.ptr,
+        _stream_ptr(stream), inp.ptr, inp.length, inp.stride, inp.type_code,
+        bins.ptr,
         bins.length, bins.type_code, locator,
         overflow.ptr if overflow is not None else None))

@@ -194,6 +194,21 @@ int32_t ilgpu_hip_radix_sort_temp_bytes(int64_t n, int32_t key_type,
   return ILGPU_HIP_SUCCESS;
 }
 
+int32_t ilgpu_hip_radix_sort_temp_bytes_strided(int64_t n, int32_t key_type,
+                                                int32_t value_bytes,
+                                                int64_t key_stride,
+                                                int64_t value_stride,
+                                                int64_t* temp_bytes) {
+  if (temp_bytes == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (key_stride < 1 || value_stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  const int32_t rc =
+      ilgpu_hip_radix_sort_temp_bytes(n, key_type, value_bytes, temp_bytes);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  *temp_bytes = radix_sort_temp_bytes(n, elem_size(key_type), value_bytes,
+                                      key_stride, value_stride);
+  return ILGPU_HIP_SUCCESS;
+}
+
 int32_t ilgpu_hip_radix_sort_keys(ilgpu_hip_stream_t stream, void* keys,
                                   int64_t n, int64_t stride, int32_t key_type,
                                   int32_t flags, void* temp,
@@ -202,12 +217,15 @@ int32_t ilgpu_hip_radix_sort_keys(ilgpu_hip_stream_t stream, void* keys,
   if (kb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (!valid_view(keys, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
   if (n > radix_sort_max_length()) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  if (stride != 1 || !aligned_to(keys, kb)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(keys, kb)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (flags & ~(ILGPU_HIP_SORT_DESCENDING | ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  const int32_t rc = check_temp(temp, temp_bytes, radix_sort_temp_bytes(n, kb, 0));
+  const int32_t rc = check_temp(temp, temp_bytes,
+                                radix_sort_temp_bytes(n, kb, 0, stride, 1));
   if (rc != ILGPU_HIP_SUCCESS) return rc;
-  SortArgs a{keys, nullptr, n, key_type, 0, flags, ILGPU_HIP_VALUES_FROM_VIEW, temp};
+  SortArgs a{keys, nullptr, stride, 1, n, key_type, 0, flags,
+             ILGPU_HIP_VALUES_FROM_VIEW, temp};
   return launch_radix_sort(static_cast<hipStream_t>(stream), a);
 }
 
@@ -224,8 +242,8 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void* keys,
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (!valid_view(keys, n) || values == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
   if (n > radix_sort_max_length()) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  if (key_stride != 1 || value_stride != 1 || !aligned_to(keys, kb) ||
-      !aligned_to(values, value_bytes))
+  if (key_stride < 1 || value_stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(keys, kb) || !aligned_to(values, value_bytes))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (flags & ~(ILGPU_HIP_SORT_DESCENDING | ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
@@ -235,10 +253,12 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void* keys,
   if (value_source == ILGPU_HIP_VALUES_FROM_INDEX && value_bytes != 4 &&
       value_bytes != 8)
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  const int32_t rc =
-      check_temp(temp, temp_bytes, radix_sort_temp_bytes(n, kb, value_bytes));
+  const int32_t rc = check_temp(
+      temp, temp_bytes,
+      radix_sort_temp_bytes(n, kb, value_bytes, key_stride, value_stride));
   if (rc != ILGPU_HIP_SUCCESS) return rc;
-  SortArgs a{keys, values, n, key_type, value_bytes, flags, value_source, temp};
+  SortArgs a{keys, values, key_stride, value_stride, n, key_type, value_bytes,
+             flags, value_source, temp};
   return launch_radix_sort(static_cast<hipStream_t>(stream), a);
 }
 
@@ -268,13 +288,13 @@ int32_t ilgpu_hip_scan(ilgpu_hip_stream_t stream, const void* in,
   if (out_length < in_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
   if (in_length > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   const int eb = elem_size(elem_type);
-  if (in_stride != 1 || out_stride != 1 || !aligned_to(in, eb) ||
-      !aligned_to(out, eb))
+  if (in_stride < 1 || out_stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(in, eb) || !aligned_to(out, eb))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   const int32_t rc = check_temp(temp, temp_bytes, scan_temp_bytes(in_length, eb));
   if (rc != ILGPU_HIP_SUCCESS) return rc;
-  return launch_scan(static_cast<hipStream_t>(stream), in, out, in_length,
-                     elem_type, op, kind, temp);
+  return launch_scan(static_cast<hipStream_t>(stream), in, in_stride, out,
+                     out_stride, in_length, elem_type, op, kind, temp);
 }
 
 /* ---- reduce ------------------------------------------------------------ */
@@ -299,12 +319,13 @@ int32_t ilgpu_hip_reduce(ilgpu_hip_stream_t stream, const void* in, int64_t n,
   if (!valid_view(out, out_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
   if (n > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   const int eb = elem_size(elem_type);
-  if (stride != 1 || !aligned_to(in, eb) || !aligned_to(out, eb))
+  if (stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(in, eb) || !aligned_to(out, eb))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   const int32_t rc = check_temp(temp, temp_bytes, reduce_temp_bytes());
   if (rc != ILGPU_HIP_SUCCESS) return rc;
-  return launch_reduce(static_cast<hipStream_t>(stream), in, n, elem_type, op,
-                       out, temp);
+  return launch_reduce(static_cast<hipStream_t>(stream), in, n, stride,
+                       elem_type, op, out, temp);
 }
 
 /* ---- histogram --------------------------------------------------------- */
@@ -325,12 +346,12 @@ int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void* in,
   if (!valid_view(in, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
   if (!valid_view(bins, num_bins)) return ILGPU_HIP_ERROR_NULL_VIEW;
   if (n > INT32_MAX || num_bins > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  if (stride != 1 || !aligned_to(in, eb) ||
-      !aligned_to(bins, elem_size(bin_type)) ||
+  if (stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(in, eb) || !aligned_to(bins, elem_size(bin_type)) ||
       (overflow != nullptr && !aligned_to(overflow, 4)))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  return launch_histogram(static_cast<hipStream_t>(stream), in, n, in_type,
-                          bins, num_bins, bin_type, locator, overflow);
+  return launch_histogram(static_cast<hipStream_t>(stream), in, n, stride,
+                          in_type, bins, num_bins, bin_type, locator, overflow);
 }
 
 }  // extern "C"

@@ -129,8 +129,8 @@ __device__ __forceinline__ bool add_to_bin_dyn(int bin_type, void* bins,
 // >= 256 bins with the identity locator).
 template <typename T, int LOC, bool RANGE_CHECK>
 __global__ __launch_bounds__(kBlock) void histogram_lds_kernel(
-    const T* __restrict__ in, int64_t n, void* bins, int num_bins, int bin_type,
-    int32_t* overflow, int replica_shift) {
+    const T* __restrict__ in, int64_t n, int64_t in_stride, void* bins,
+    int num_bins, int bin_type, int32_t* overflow, int replica_shift) {
   using V = typename Vec16<T>::type;
   constexpr int VN = Vec16<T>::N;
   extern __shared__ uint32_t s_counts[];
@@ -152,11 +152,19 @@ __global__ __launch_bounds__(kBlock) void histogram_lds_kernel(
   int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(T));
   if (head > n) head = n;
   const V* body = reinterpret_cast<const V*>(in + head);
-  const int64_t nvec = (n - head) / VN;
-  const int64_t tail_start = head + nvec * VN;
+  int64_t nvec = (n - head) / VN;
+  int64_t tail_start = head + nvec * VN;
 
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (in_stride != 1) {
+    // Stride1D.General with an element stride above one: sample i lives at
+    // in[i * in_stride]; one scalar load per sample, no vector body.
+    for (int64_t e = i; e < n; e += stride) count(in[e * in_stride]);
+    nvec = 0;
+    head = 0;
+    tail_start = n;
+  }
   for (; i + (kUnroll - 1) * stride < nvec; i += kUnroll * stride) {
     V v[kUnroll];
 #pragma unroll
@@ -205,14 +213,14 @@ __global__ __launch_bounds__(kBlock) void histogram_lds_kernel(
 // More bins than LDS holds: one global atomic per element, as the reference.
 template <typename T, int LOC>
 __global__ __launch_bounds__(kBlock) void histogram_global_kernel(
-    const T* __restrict__ in, int64_t n, void* bins, int64_t num_bins,
-    int bin_type, int32_t* overflow) {
+    const T* __restrict__ in, int64_t n, int64_t in_stride, void* bins,
+    int64_t num_bins, int bin_type, int32_t* overflow) {
   const bool checked = overflow != nullptr;
   bool passed = false;
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
        i += stride) {
-    const int64_t b = locate<T, LOC>(in[i], (int)num_bins);
+    const int64_t b = locate<T, LOC>(in[i * in_stride], (int)num_bins);
     if ((uint64_t)b < (uint64_t)num_bins)
       passed |= add_to_bin_dyn(bin_type, bins, b, 1u, checked);
   }
@@ -234,8 +242,9 @@ template <> constexpr double type_max_as_double<float>() { return 3.5e38; }
 template <> constexpr double type_max_as_double<double>() { return 1.7e308; }
 
 template <typename T, int LOC>
-int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* bins,
-                     int64_t num_bins, int32_t bin_type, int32_t* overflow) {
+int32_t launch_typed(hipStream_t stream, const void* in, int64_t n,
+                     int64_t in_stride, void* bins, int64_t num_bins,
+                     int32_t bin_type, int32_t* overflow) {
   const T* src = static_cast<const T*>(in);
   const int cus = device_cu_count();
   ProfileScope scope(stream, "histogram");
@@ -243,8 +252,8 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* bins,
     int64_t blocks = div_up(n, kBlock);
     if (blocks > (int64_t)cus * 4) blocks = (int64_t)cus * 4;
     hipLaunchKernelGGL((histogram_global_kernel<T, LOC>), dim3((unsigned)blocks),
-                       dim3(kBlock), 0, stream, src, n, bins, num_bins,
-                       bin_type, overflow);
+                       dim3(kBlock), 0, stream, src, n, in_stride, bins,
+                       num_bins, bin_type, overflow);
     ILGPU_HIP_CHECK(hipGetLastError());
     return ILGPU_HIP_SUCCESS;
   }
@@ -269,11 +278,13 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* bins,
   if (no_check) {
     hipLaunchKernelGGL((histogram_lds_kernel<T, LOC, false>),
                        dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream,
-                       src, n, bins, (int)num_bins, bin_type, overflow, shift);
+                       src, n, in_stride, bins, (int)num_bins, bin_type, overflow,
+                       shift);
   } else {
     hipLaunchKernelGGL((histogram_lds_kernel<T, LOC, true>),
                        dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream,
-                       src, n, bins, (int)num_bins, bin_type, overflow, shift);
+                       src, n, in_stride, bins, (int)num_bins, bin_type, overflow,
+                       shift);
   }
   ILGPU_HIP_CHECK(hipGetLastError());
   return ILGPU_HIP_SUCCESS;
@@ -281,15 +292,15 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* bins,
 
 template <typename T>
 int32_t launch_locator(hipStream_t stream, const void* in, int64_t n,
-                       void* bins, int64_t num_bins, int32_t bin_type,
-                       int32_t locator, int32_t* overflow) {
+                       int64_t in_stride, void* bins, int64_t num_bins,
+                       int32_t bin_type, int32_t locator, int32_t* overflow) {
   switch (locator) {
     case ILGPU_HIP_LOCATOR_IDENTITY:
       return launch_typed<T, ILGPU_HIP_LOCATOR_IDENTITY>(
-          stream, in, n, bins, num_bins, bin_type, overflow);
+          stream, in, n, in_stride, bins, num_bins, bin_type, overflow);
     case ILGPU_HIP_LOCATOR_MODULO:
       return launch_typed<T, ILGPU_HIP_LOCATOR_MODULO>(
-          stream, in, n, bins, num_bins, bin_type, overflow);
+          stream, in, n, in_stride, bins, num_bins, bin_type, overflow);
     default:
       return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
@@ -298,12 +309,13 @@ int32_t launch_locator(hipStream_t stream, const void* in, int64_t n,
 }  // namespace
 
 int32_t launch_histogram(hipStream_t stream, const void* in, int64_t n,
-                         int32_t in_type, void* bins, int64_t num_bins,
-                         int32_t bin_type, int32_t locator, int32_t* overflow) {
+                         int64_t in_stride, int32_t in_type, void* bins,
+                         int64_t num_bins, int32_t bin_type, int32_t locator,
+                         int32_t* overflow) {
 #define ILGPU_HIP_HIST_CASE(CODE, T)                                      \
   case CODE:                                                              \
-    return launch_locator<T>(stream, in, n, bins, num_bins, bin_type,     \
-                             locator, overflow)
+    return launch_locator<T>(stream, in, n, in_stride, bins, num_bins,    \
+                             bin_type, locator, overflow)
   switch (in_type) {
     ILGPU_HIP_HIST_CASE(ILGPU_HIP_I8, int8_t);
     ILGPU_HIP_HIST_CASE(ILGPU_HIP_I16, int16_t);

@@ -1,6 +1,7 @@
 // Internal launch interface between the C ABI (api.hip) and the kernel files.
 // All launchers assume validated arguments: non-null, naturally aligned
-// device pointers, 1 <= n <= INT32_MAX, stride 1, temp large enough.
+// device pointers, 1 <= n <= INT32_MAX, element strides >= 1, temp large
+// enough.
 #pragma once
 
 #include "common.hpp"
@@ -10,22 +11,27 @@ namespace ilgpu_hip {
 // reduce.hip
 int64_t reduce_temp_bytes();
 int32_t launch_reduce(hipStream_t stream, const void* in, int64_t n,
-                      int32_t type, int32_t op, void* out, void* temp);
+                      int64_t in_stride, int32_t type, int32_t op, void* out,
+                      void* temp);
 
 // scan.hip
 int64_t scan_temp_bytes(int64_t n, int elem_bytes);
-int32_t launch_scan(hipStream_t stream, const void* in, void* out, int64_t n,
-                    int32_t type, int32_t op, int32_t kind, void* temp);
+int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
+                    void* out, int64_t out_stride, int64_t n, int32_t type,
+                    int32_t op, int32_t kind, void* temp);
 
 // histogram.hip
 int32_t launch_histogram(hipStream_t stream, const void* in, int64_t n,
-                         int32_t in_type, void* bins, int64_t num_bins,
-                         int32_t bin_type, int32_t locator, int32_t* overflow);
+                         int64_t in_stride, int32_t in_type, void* bins,
+                         int64_t num_bins, int32_t bin_type, int32_t locator,
+                         int32_t* overflow);
 
 // radix_sort.hip
 struct SortArgs {
   void* keys;
   void* values;      // nullptr for a keys-only sort
+  int64_t key_stride;    // element strides of the two views
+  int64_t value_stride;
   int64_t n;
   int32_t key_type;
   int32_t value_bytes;   // 0 for keys only
@@ -33,7 +39,9 @@ struct SortArgs {
   int32_t value_source;
   void* temp;
 };
-int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes);
+// Strides above one add a dense staging copy of that view to the temp.
+int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
+                              int64_t key_stride = 1, int64_t value_stride = 1);
 int64_t radix_sort_max_length();
 int32_t launch_radix_sort(hipStream_t stream, const SortArgs& args);
 

@@ -761,15 +761,58 @@ int32_t launch_value(hipStream_t stream, const SortArgs& a) {
   }
 }
 
-}  // namespace
-
-int64_t radix_sort_max_length() { return kMaxSortLength; }
-
-int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes) {
-  return 256 + make_layout(n, key_bytes, value_bytes).total;
+// ---- strided views ------------------------------------------------------------
+// Stride1D.General with an element stride above one: the view is gathered
+// into a dense staging copy behind the dense sort's temp area, sorted there
+// and scattered back; elements between the strided ones are never touched.
+template <typename E>
+__global__ __launch_bounds__(256) void gather_strided_kernel(
+    const E* __restrict__ src, int64_t stride, E* __restrict__ dst, int64_t n) {
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
+    dst[i] = src[i * stride];
 }
 
-int32_t launch_radix_sort(hipStream_t stream, const SortArgs& a) {
+template <typename E>
+__global__ __launch_bounds__(256) void scatter_strided_kernel(
+    const E* __restrict__ src, E* __restrict__ dst, int64_t stride, int64_t n) {
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
+    dst[i * stride] = src[i];
+}
+
+template <typename E>
+int32_t copy_strided(hipStream_t stream, bool gather, void* strided, int64_t stride,
+                     void* dense, int64_t n) {
+  int64_t blocks = div_up(n, 256);
+  const int64_t cap = (int64_t)device_cu_count() * 8;
+  if (blocks > cap) blocks = cap;
+  ProfileScope scope(stream, gather ? "sort_gather" : "sort_scatter");
+  if (gather)
+    hipLaunchKernelGGL((gather_strided_kernel<E>), dim3((unsigned)blocks), dim3(256), 0,
+                       stream, static_cast<const E*>(strided), stride,
+                       static_cast<E*>(dense), n);
+  else
+    hipLaunchKernelGGL((scatter_strided_kernel<E>), dim3((unsigned)blocks), dim3(256), 0,
+                       stream, static_cast<const E*>(dense), static_cast<E*>(strided),
+                       stride, n);
+  ILGPU_HIP_CHECK(hipGetLastError());
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t copy_strided_bytes(hipStream_t stream, bool gather, int elem_bytes, void* strided,
+                           int64_t stride, void* dense, int64_t n) {
+  switch (elem_bytes) {
+    case 1: return copy_strided<uint8_t>(stream, gather, strided, stride, dense, n);
+    case 2: return copy_strided<uint16_t>(stream, gather, strided, stride, dense, n);
+    case 4: return copy_strided<uint32_t>(stream, gather, strided, stride, dense, n);
+    case 8: return copy_strided<uint64_t>(stream, gather, strided, stride, dense, n);
+    case 16: return copy_strided<Bytes16>(stream, gather, strided, stride, dense, n);
+    default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  }
+}
+
+int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
   switch (elem_size(a.key_type)) {
     case 1: return launch_value<1>(stream, a);
     case 2: return launch_value<2>(stream, a);
@@ -777,6 +820,60 @@ int32_t launch_radix_sort(hipStream_t stream, const SortArgs& a) {
     case 8: return launch_value<8>(stream, a);
     default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
+}
+
+}  // namespace
+
+int64_t radix_sort_max_length() { return kMaxSortLength; }
+
+int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
+                              int64_t key_stride, int64_t value_stride) {
+  int64_t total = 256 + make_layout(n, key_bytes, value_bytes).total;
+  if (key_stride != 1 || (value_bytes > 0 && value_stride != 1)) {
+    total = align_up(total, 256);
+    if (key_stride != 1) total += align_up(n * key_bytes, 256);
+    if (value_bytes > 0 && value_stride != 1) total += align_up(n * value_bytes, 256);
+  }
+  return total;
+}
+
+int32_t launch_radix_sort(hipStream_t stream, const SortArgs& a) {
+  const bool has_values = a.values != nullptr && a.value_bytes > 0;
+  const bool keys_strided = a.key_stride != 1;
+  const bool values_strided = has_values && a.value_stride != 1;
+  if (!keys_strided && !values_strided) return launch_dense(stream, a);
+
+  const int kb = elem_size(a.key_type);
+  char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)a.temp, 256));
+  char* staging = base + align_up(make_layout(a.n, kb, a.value_bytes).total, 256);
+  SortArgs dense = a;
+  dense.key_stride = 1;
+  dense.value_stride = 1;
+  int32_t rc;
+  if (keys_strided) {
+    dense.keys = staging;
+    staging += align_up(a.n * kb, 256);
+    rc = copy_strided_bytes(stream, true, kb, a.keys, a.key_stride, dense.keys, a.n);
+    if (rc != ILGPU_HIP_SUCCESS) return rc;
+  }
+  if (values_strided) {
+    dense.values = staging;
+    if (a.value_source == ILGPU_HIP_VALUES_FROM_VIEW) {
+      rc = copy_strided_bytes(stream, true, a.value_bytes, a.values, a.value_stride,
+                              dense.values, a.n);
+      if (rc != ILGPU_HIP_SUCCESS) return rc;
+    }
+  }
+  rc = launch_dense(stream, dense);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  if (keys_strided) {
+    rc = copy_strided_bytes(stream, false, kb, a.keys, a.key_stride, dense.keys, a.n);
+    if (rc != ILGPU_HIP_SUCCESS) return rc;
+  }
+  if (values_strided)
+    rc = copy_strided_bytes(stream, false, a.value_bytes, a.values, a.value_stride,
+                            dense.values, a.n);
+  return rc;
 }
 
 }  // namespace ilgpu_hip

@@ -59,13 +59,25 @@ __device__ __forceinline__ A block_fold(A v, A* lds) {
 
 template <typename T, int OP>
 __global__ __launch_bounds__(kBlock) void reduce_partials_kernel(
-    const T* __restrict__ in, int64_t n,
+    const T* __restrict__ in, int64_t n, int64_t in_stride,
     typename AccType<T, OP>::type* __restrict__ partials) {
   using A = typename AccType<T, OP>::type;
   using F = Functor<A, OP>;
   using V = typename Vec16<T>::type;
   constexpr int VN = Vec16<T>::N;
   __shared__ A lds[kBlock / kWaveSize];
+
+  if (in_stride != 1) {
+    // Stride1D.General with an element stride above one: element i lives at
+    // in[i * in_stride]; one scalar load per element.
+    A acc = F::identity();
+    const int64_t step = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step)
+      acc = F::apply(acc, (A)in[i * in_stride]);
+    A r = block_fold<A, OP>(acc, lds);
+    if (threadIdx.x == 0) partials[blockIdx.x] = r;
+    return;
+  }
 
   // Split [0,n) into an unaligned head, a body of whole 16-byte vectors and a
   // tail; head and tail together hold fewer than 2*VN elements.
@@ -127,8 +139,8 @@ __global__ __launch_bounds__(kBlock) void reduce_final_kernel(
 }
 
 template <typename T, int OP>
-int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* out,
-                     void* temp) {
+int32_t launch_typed(hipStream_t stream, const void* in, int64_t n,
+                     int64_t in_stride, void* out, void* temp) {
   using A = typename AccType<T, OP>::type;
   const int64_t nvec = n / Vec16<T>::N;
   int64_t blocks = div_up(nvec > 0 ? nvec : 1, kBlock);
@@ -141,7 +153,7 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* out,
     ProfileScope scope(stream, "reduce_partials");
     hipLaunchKernelGGL((reduce_partials_kernel<T, OP>), dim3((unsigned)blocks),
                        dim3(kBlock), 0, stream, static_cast<const T*>(in), n,
-                       partials);
+                       in_stride, partials);
   }
   ILGPU_HIP_CHECK(hipGetLastError());
   {
@@ -154,15 +166,15 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n, void* out,
 }
 
 template <typename T>
-int32_t launch_op(hipStream_t stream, const void* in, int64_t n, int32_t op,
-                  void* out, void* temp) {
+int32_t launch_op(hipStream_t stream, const void* in, int64_t n,
+                  int64_t in_stride, int32_t op, void* out, void* temp) {
   switch (op) {
     case ILGPU_HIP_OP_ADD:
-      return launch_typed<T, ILGPU_HIP_OP_ADD>(stream, in, n, out, temp);
+      return launch_typed<T, ILGPU_HIP_OP_ADD>(stream, in, n, in_stride, out, temp);
     case ILGPU_HIP_OP_MAX:
-      return launch_typed<T, ILGPU_HIP_OP_MAX>(stream, in, n, out, temp);
+      return launch_typed<T, ILGPU_HIP_OP_MAX>(stream, in, n, in_stride, out, temp);
     case ILGPU_HIP_OP_MIN:
-      return launch_typed<T, ILGPU_HIP_OP_MIN>(stream, in, n, out, temp);
+      return launch_typed<T, ILGPU_HIP_OP_MIN>(stream, in, n, in_stride, out, temp);
     default:
       return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
@@ -173,14 +185,15 @@ int32_t launch_op(hipStream_t stream, const void* in, int64_t n, int32_t op,
 int64_t reduce_temp_bytes() { return (int64_t)kMaxBlocks * 8 + 16; }
 
 int32_t launch_reduce(hipStream_t stream, const void* in, int64_t n,
-                      int32_t type, int32_t op, void* out, void* temp) {
+                      int64_t in_stride, int32_t type, int32_t op, void* out,
+                      void* temp) {
   switch (type) {
-    case ILGPU_HIP_I32: return launch_op<int32_t>(stream, in, n, op, out, temp);
-    case ILGPU_HIP_U32: return launch_op<uint32_t>(stream, in, n, op, out, temp);
-    case ILGPU_HIP_I64: return launch_op<int64_t>(stream, in, n, op, out, temp);
-    case ILGPU_HIP_U64: return launch_op<uint64_t>(stream, in, n, op, out, temp);
-    case ILGPU_HIP_F32: return launch_op<float>(stream, in, n, op, out, temp);
-    case ILGPU_HIP_F64: return launch_op<double>(stream, in, n, op, out, temp);
+    case ILGPU_HIP_I32: return launch_op<int32_t>(stream, in, n, in_stride, op, out, temp);
+    case ILGPU_HIP_U32: return launch_op<uint32_t>(stream, in, n, in_stride, op, out, temp);
+    case ILGPU_HIP_I64: return launch_op<int64_t>(stream, in, n, in_stride, op, out, temp);
+    case ILGPU_HIP_U64: return launch_op<uint64_t>(stream, in, n, in_stride, op, out, temp);
+    case ILGPU_HIP_F32: return launch_op<float>(stream, in, n, in_stride, op, out, temp);
+    case ILGPU_HIP_F64: return launch_op<double>(stream, in, n, in_stride, op, out, temp);
     default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
 }

@@ -171,7 +171,8 @@ __device__ __forceinline__ T resolve_prefix(const TileState<T>& st, int tile,
 
 template <typename T, int OP, bool VECTOR>
 __global__ __launch_bounds__(kBlock) void scan_kernel(
-    const T* __restrict__ in, T* __restrict__ out, int64_t n, int inclusive,
+    const T* __restrict__ in, T* __restrict__ out, int64_t n,
+    int64_t in_stride, int64_t out_stride, int inclusive,
     uint32_t* __restrict__ ticket, TileState<T> st) {
   using F = Functor<T, OP>;
   using V = typename Vec16<T>::type;
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
         const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
-        x[j][k] = idx < n ? in[idx] : F::identity();
+        x[j][k] = idx < n ? in[idx * in_stride] : F::identity();
       }
   }
 
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
         const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
-        if (idx < n) out[idx] = r[k];
+        if (idx < n) out[idx * out_stride] = r[k];
       }
     }
     running = F::apply(running, seg_total[j]);
@@ -282,8 +283,9 @@ template <typename T> int64_t num_tiles(int64_t n) {
 }
 
 template <typename T, int OP>
-int32_t launch_typed(hipStream_t stream, const void* in, void* out, int64_t n,
-                     int32_t kind, void* temp) {
+int32_t launch_typed(hipStream_t stream, const void* in, int64_t in_stride,
+                     void* out, int64_t out_stride, int64_t n, int32_t kind,
+                     void* temp) {
   const int64_t tiles = num_tiles<T>(n);
   char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)temp, 256));
   uint32_t* ticket = reinterpret_cast<uint32_t*>(base);
@@ -302,33 +304,41 @@ int32_t launch_typed(hipStream_t stream, const void* in, void* out, int64_t n,
   int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
                                  zero_words);
   if (rc != ILGPU_HIP_SUCCESS) return rc;
-  const bool vector = (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
+  // Element strides above one (Stride1D.General) take the scalar path.
+  const bool vector = in_stride == 1 && out_stride == 1 &&
+                      (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
                       (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   const int inclusive = kind == ILGPU_HIP_SCAN_INCLUSIVE ? 1 : 0;
   ProfileScope scope(stream, "scan");
   if (vector) {
     hipLaunchKernelGGL((scan_kernel<T, OP, true>), dim3((unsigned)tiles),
                        dim3(kBlock), 0, stream, static_cast<const T*>(in),
-                       static_cast<T*>(out), n, inclusive, ticket, st);
+                       static_cast<T*>(out), n, in_stride, out_stride,
+                       inclusive, ticket, st);
   } else {
     hipLaunchKernelGGL((scan_kernel<T, OP, false>), dim3((unsigned)tiles),
                        dim3(kBlock), 0, stream, static_cast<const T*>(in),
-                       static_cast<T*>(out), n, inclusive, ticket, st);
+                       static_cast<T*>(out), n, in_stride, out_stride,
+                       inclusive, ticket, st);
   }
   ILGPU_HIP_CHECK(hipGetLastError());
   return ILGPU_HIP_SUCCESS;
 }
 
 template <typename T>
-int32_t launch_op(hipStream_t stream, const void* in, void* out, int64_t n,
-                  int32_t op, int32_t kind, void* temp) {
+int32_t launch_op(hipStream_t stream, const void* in, int64_t in_stride,
+                  void* out, int64_t out_stride, int64_t n, int32_t op,
+                  int32_t kind, void* temp) {
   switch (op) {
     case ILGPU_HIP_OP_ADD:
-      return launch_typed<T, ILGPU_HIP_OP_ADD>(stream, in, out, n, kind, temp);
+      return launch_typed<T, ILGPU_HIP_OP_ADD>(stream, in, in_stride, out, out_stride, n,
+                                               kind, temp);
     case ILGPU_HIP_OP_MAX:
-      return launch_typed<T, ILGPU_HIP_OP_MAX>(stream, in, out, n, kind, temp);
+      return launch_typed<T, ILGPU_HIP_OP_MAX>(stream, in, in_stride, out, out_stride, n,
+                                               kind, temp);
     case ILGPU_HIP_OP_MIN:
-      return launch_typed<T, ILGPU_HIP_OP_MIN>(stream, in, out, n, kind, temp);
+      return launch_typed<T, ILGPU_HIP_OP_MIN>(stream, in, in_stride, out, out_stride, n,
+                                               kind, temp);
     default:
       return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
@@ -357,15 +367,16 @@ int64_t scan_temp_bytes(int64_t n, int elem_bytes) {
   return 256 + kHeaderBytes + align_up(tiles * 4, 256) + tiles * 16;
 }
 
-int32_t launch_scan(hipStream_t stream, const void* in, void* out, int64_t n,
-                    int32_t type, int32_t op, int32_t kind, void* temp) {
+int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
+                    void* out, int64_t out_stride, int64_t n, int32_t type,
+                    int32_t op, int32_t kind, void* temp) {
   switch (type) {
-    case ILGPU_HIP_I32: return launch_op<int32_t>(stream, in, out, n, op, kind, temp);
-    case ILGPU_HIP_U32: return launch_op<uint32_t>(stream, in, out, n, op, kind, temp);
-    case ILGPU_HIP_I64: return launch_op<int64_t>(stream, in, out, n, op, kind, temp);
-    case ILGPU_HIP_U64: return launch_op<uint64_t>(stream, in, out, n, op, kind, temp);
-    case ILGPU_HIP_F32: return launch_op<float>(stream, in, out, n, op, kind, temp);
-    case ILGPU_HIP_F64: return launch_op<double>(stream, in, out, n, op, kind, temp);
+    case ILGPU_HIP_I32: return launch_op<int32_t>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
+    case ILGPU_HIP_U32: return launch_op<uint32_t>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
+    case ILGPU_HIP_I64: return launch_op<int64_t>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
+    case ILGPU_HIP_U64: return launch_op<uint64_t>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
+    case ILGPU_HIP_F32: return launch_op<float>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
+    case ILGPU_HIP_F64: return launch_op<double>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
     default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
 }

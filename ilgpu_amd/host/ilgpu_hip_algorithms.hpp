@@ -321,10 +321,6 @@ inline Index1D BytesToInts(int64_t bytes) {
   return (Index1D)ints;
 }
 
-inline void RequireDense(int64_t stride) {
-  if (stride != 1) throw NotSupportedException("only stride 1 views are supported");
-}
-
 // ---- radix sort (RadixSortExtensions.cs) ---------------------------------------
 template <typename T, typename TStride>
 using RadixSort = std::function<void(AcceleratorStream&, ArrayView1D<T, TStride>, ArrayView<int32_t>)>;
@@ -343,6 +339,28 @@ Index1D ComputeRadixSortTempStorageSize(Accelerator&, Index1D dataLength) {
   int64_t bytes = 0;
   HipAlgorithmsException::ThrowIfFailed(
       ilgpu_hip_radix_sort_temp_bytes(dataLength, TypeCode<T>::value, 0, &bytes), "dataLength");
+  return BytesToInts(bytes);
+}
+// The same for a Stride1D.General view with an element stride above one: the
+// sort stages a dense copy of the view in the temp.  The reference has no such
+// overload (its kernels index through the view); passing the dense size for a
+// strided view throws ArgumentOutOfRangeException("tempView").
+template <typename T, typename TRadixSortOperation>
+Index1D ComputeRadixSortTempStorageSize(Accelerator&, Index1D dataLength, int64_t stride) {
+  int64_t bytes = 0;
+  HipAlgorithmsException::ThrowIfFailed(
+      ilgpu_hip_radix_sort_temp_bytes_strided(dataLength, TypeCode<T>::value, 0, stride, 1,
+                                              &bytes), "dataLength");
+  return BytesToInts(bytes);
+}
+template <typename TKey, typename TValue, typename TRadixSortOperation>
+Index1D ComputeRadixSortPairsTempStorageSize(Accelerator&, Index1D dataLength,
+                                             int64_t keyStride, int64_t valueStride) {
+  int64_t bytes = 0;
+  HipAlgorithmsException::ThrowIfFailed(
+      ilgpu_hip_radix_sort_temp_bytes_strided(dataLength, TypeCode<TKey>::value,
+                                              (int32_t)sizeof(TValue), keyStride,
+                                              valueStride, &bytes), "dataLength");
   return BytesToInts(bytes);
 }
 // ComputeRadixSortPairsTempStorageSize (:384-404); sized in 64-bit bytes first.
@@ -367,12 +385,11 @@ RadixSort<T, TStride> CreateRadixSort(Accelerator&) {
     if (!input.IsValid()) throw ArgumentNullException("input");
     if (input.Length() > std::numeric_limits<int32_t>::max())
       throw NotSupportedException("NotSupportedArrayView64");
-    RequireDense(input.Stride().Stride());
     TempViewManager viewManager(tempView, "tempView");
     HipAlgorithmsException::ThrowIfFailed(
         ilgpu_hip_radix_sort_keys(
-            stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(), 1,
-            TypeCode<T>::value,
+            stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(),
+            input.Stride().Stride(), TypeCode<T>::value,
             TRadixSortOperation::Descending ? ILGPU_HIP_SORT_DESCENDING : 0,
             tempView.LoadEffectiveAddressAsPtr(), tempView.Length() * 4),
         "tempView");
@@ -390,13 +407,12 @@ RadixSortPairs<TKey, TKeyStride, TValue, TValueStride> CreateRadixSortPairs(Acce
     if (!keys.IsValid()) throw ArgumentNullException("keys");
     if (!values.IsValid()) throw ArgumentNullException("values");
     if (keys.Length() != values.Length()) throw ArgumentOutOfRangeException("values");
-    RequireDense(keys.Stride().Stride());
-    RequireDense(values.Stride().Stride());
     TempViewManager viewManager(tempView, "tempView");
     HipAlgorithmsException::ThrowIfFailed(
         ilgpu_hip_radix_sort_pairs(
-            stream.StreamPtr(), keys.LoadEffectiveAddressAsPtr(), 1,
-            values.LoadEffectiveAddressAsPtr(), 1, keys.Length(), TypeCode<TKey>::value,
+            stream.StreamPtr(), keys.LoadEffectiveAddressAsPtr(), keys.Stride().Stride(),
+            values.LoadEffectiveAddressAsPtr(), values.Stride().Stride(), keys.Length(),
+            TypeCode<TKey>::value,
             (int32_t)sizeof(TValue),
             TRadixSortOperation::Descending ? ILGPU_HIP_SORT_DESCENDING : 0,
             ILGPU_HIP_VALUES_FROM_VIEW, tempView.LoadEffectiveAddressAsPtr(),
@@ -422,8 +438,9 @@ CreateRadixSortPairsWithSequencer(Accelerator&) {
     TempViewManager viewManager(tempView, "tempView");
     HipAlgorithmsException::ThrowIfFailed(
         ilgpu_hip_radix_sort_pairs(
-            stream.StreamPtr(), keys.LoadEffectiveAddressAsPtr(), 1,
-            values.LoadEffectiveAddressAsPtr(), 1, keys.Length(), TypeCode<TKey>::value,
+            stream.StreamPtr(), keys.LoadEffectiveAddressAsPtr(), keys.Stride().Stride(),
+            values.LoadEffectiveAddressAsPtr(), values.Stride().Stride(), keys.Length(),
+            TypeCode<TKey>::value,
             (int32_t)sizeof(TValue),
             TRadixSortOperation::Descending ? ILGPU_HIP_SORT_DESCENDING : 0,
             ILGPU_HIP_VALUES_FROM_INDEX, tempView.LoadEffectiveAddressAsPtr(),
@@ -500,12 +517,11 @@ Scan<T, TStrideIn, TStrideOut> CreateScan(Accelerator&, ScanKind kind) {
     if (output.Length() < input.Length()) throw ArgumentOutOfRangeException("output");
     if (input.Length() > std::numeric_limits<int32_t>::max())
       throw NotSupportedException("NotSupportedArrayView64");
-    RequireDense(input.Stride().Stride());
-    RequireDense(output.Stride().Stride());
     TempViewManager viewManager(temp, "temp");
     HipAlgorithmsException::ThrowIfFailed(
-        ilgpu_hip_scan(stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(), 1,
-                       output.LoadEffectiveAddressAsPtr(), output.Length(), 1,
+        ilgpu_hip_scan(stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(),
+                       input.Stride().Stride(), output.LoadEffectiveAddressAsPtr(),
+                       output.Length(), output.Stride().Stride(),
                        TypeCode<T>::value, TScanOperation::Op, (int32_t)kind,
                        temp.LoadEffectiveAddressAsPtr(), temp.Length() * 4),
         "temp");
@@ -558,9 +574,9 @@ Reduction<T, TStride> CreateReduction(Accelerator& accelerator) {
     if (input.Length() < 1) throw ArgumentOutOfRangeException("input");
     if (!output.IsValid()) throw ArgumentNullException("output");
     if (output.Length() < 1) throw ArgumentOutOfRangeException("output");
-    RequireDense(input.Stride().Stride());
     HipAlgorithmsException::ThrowIfFailed(
-        ilgpu_hip_reduce(stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(), 1,
+        ilgpu_hip_reduce(stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(),
+                         input.Stride().Stride(),
                          TypeCode<T>::value, TReduction::Op,
                          output.LoadEffectiveAddressAsPtr(), output.Length(),
                          scratch->View().LoadEffectiveAddressAsPtr(),
@@ -606,9 +622,9 @@ HistogramDelegate<T, TStride, TBinType> CreateHistogram(Accelerator&) {
     if (view.Length() > std::numeric_limits<int32_t>::max() ||
         histogram.Length() > std::numeric_limits<int32_t>::max())
       throw NotSupportedException("NotSupportedArrayView64");
-    RequireDense(view.Stride().Stride());
     HipAlgorithmsException::ThrowIfFailed(
-        ilgpu_hip_histogram(stream.StreamPtr(), view.LoadEffectiveAddressAsPtr(), view.Length(), 1,
+        ilgpu_hip_histogram(stream.StreamPtr(), view.LoadEffectiveAddressAsPtr(), view.Length(),
+                            view.Stride().Stride(),
                             TypeCode<T>::value, histogram.LoadEffectiveAddressAsPtr(),
                             histogram.Length(), TypeCode<TBinType>::value, TLocator::Locator,
                             histogramOverflow.LoadEffectiveAddressAsPtr()),
@@ -625,9 +641,9 @@ HistogramUncheckedDelegate<T, TStride, TBinType> CreateHistogramUnchecked(Accele
     if (view.Length() > std::numeric_limits<int32_t>::max() ||
         histogram.Length() > std::numeric_limits<int32_t>::max())
       throw NotSupportedException("NotSupportedArrayView64");
-    RequireDense(view.Stride().Stride());
     HipAlgorithmsException::ThrowIfFailed(
-        ilgpu_hip_histogram(stream.StreamPtr(), view.LoadEffectiveAddressAsPtr(), view.Length(), 1,
+        ilgpu_hip_histogram(stream.StreamPtr(), view.LoadEffectiveAddressAsPtr(), view.Length(),
+                            view.Stride().Stride(),
                             TypeCode<T>::value, histogram.LoadEffectiveAddressAsPtr(),
                             histogram.Length(), TypeCode<TBinType>::value, TLocator::Locator,
                             nullptr),

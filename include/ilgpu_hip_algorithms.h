@@ -15,9 +15,13 @@
  *  - `stream` is a hipStream_t (NULL = the default stream).  All work is
  *    enqueued asynchronously on it, like the reference's delegates; the
  *    caller synchronises before reading results.
- *  - Lengths and strides count ELEMENTS.  Only stride == 1 (Stride1D.Dense,
- *    or Stride1D.General with stride 1 as the reference's tests use) is
- *    accepted; anything else returns ILGPU_HIP_ERROR_NOT_SUPPORTED.
+ *  - Lengths and strides count ELEMENTS: element i of a view is at
+ *    base[i * stride] (ArrayView1D<T, Stride1D.General>, ArrayViews.tt:114-119;
+ *    Stride1D.Dense is stride 1).  Stride 1 takes the vectorised kernels;
+ *    larger strides are served by scalar loads and stores (scan, reduce,
+ *    histogram) or by a dense staging copy in temp (sort), and elements
+ *    between the strided ones are never read or written.  Strides below 1
+ *    return ILGPU_HIP_ERROR_OUT_OF_RANGE.
  *  - Lengths above INT32_MAX return ILGPU_HIP_ERROR_NOT_SUPPORTED, like
  *    ErrorMessages.NotSupportedArrayView64 in the reference.
  *  - The library allocates no device memory and keeps no pointer after a call
@@ -135,6 +139,18 @@ int32_t ilgpu_hip_profile_query(const char *kernel_name, int64_t *launches,
 int32_t ilgpu_hip_radix_sort_temp_bytes(int64_t n, int32_t key_type,
                                         int32_t value_bytes,
                                         int64_t *temp_bytes);
+
+/* The same for views with element strides above one: each strided view adds a
+ * dense staging copy of its n elements.  ComputeRadixSortTempStorageSize has no
+ * stride argument (RadixSortExtensions.cs:419-447: the reference's kernels
+ * index through the view), so a binding offers this as an overload that takes
+ * the views' strides; sorting a strided view with the dense size returns
+ * ILGPU_HIP_ERROR_OUT_OF_RANGE (temp too small). */
+int32_t ilgpu_hip_radix_sort_temp_bytes_strided(int64_t n, int32_t key_type,
+                                                int32_t value_bytes,
+                                                int64_t key_stride,
+                                                int64_t value_stride,
+                                                int64_t *temp_bytes);
 
 int32_t ilgpu_hip_radix_sort_keys(ilgpu_hip_stream_t stream, void *keys,
                                   int64_t n, int64_t stride, int32_t key_type,

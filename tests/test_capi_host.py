@@ -80,9 +80,17 @@ def test_sort_argument_validation():
     assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 0, FAKE, 8) == capi.ERROR_OUT_OF_RANGE
     # temp not int-aligned -> InvalidOperationException
     assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 0, FAKE + 2, big) == capi.ERROR_UNALIGNED_TEMP
-    # 64-bit lengths, strides, unknown types/flags -> NotSupportedException
+    # 64-bit lengths, unknown types/flags -> NotSupportedException
     assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 1 << 31, 1, capi.U32, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
-    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 2, capi.U32, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    # strides below one; a strided view with the dense temp size (too small)
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 0, capi.U32, 0, FAKE, big) == capi.ERROR_OUT_OF_RANGE
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, -2, capi.U32, 0, FAKE, big) == capi.ERROR_OUT_OF_RANGE
+    dense = capi.radix_sort_temp_bytes(16, np.uint32)
+    assert capi.radix_sort_temp_bytes(16, np.uint32, 0, 3) >= dense + 16 * 4
+    assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 3, capi.U32, 0, FAKE, dense) == capi.ERROR_OUT_OF_RANGE
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 0, 16, capi.U32, 4, 0, 0, FAKE, big) == capi.ERROR_OUT_OF_RANGE
+    assert (capi.radix_sort_temp_bytes(16, np.uint32, 8, 1, 5)
+            >= capi.radix_sort_temp_bytes(16, np.uint32, 8) + 16 * 8)
     assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, 42, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
     assert L.ilgpu_hip_radix_sort_keys(None, FAKE, 16, 1, capi.U32, 8, FAKE, big) == capi.ERROR_NOT_SUPPORTED
     # pairs
@@ -107,7 +115,8 @@ def test_scan_argument_validation():
     assert call(n_in=0) == capi.ERROR_NULL_VIEW
     assert call(n_out=8) == capi.ERROR_OUT_OF_RANGE        # ScanExtensions.cs:679-680
     assert call(n_in=1 << 31, n_out=1 << 31) == capi.ERROR_NOT_SUPPORTED
-    assert call(s_in=2) == capi.ERROR_NOT_SUPPORTED
+    assert call(s_in=0) == capi.ERROR_OUT_OF_RANGE
+    assert call(s_out=-1) == capi.ERROR_OUT_OF_RANGE
     assert call(t=capi.U8) == capi.ERROR_NOT_SUPPORTED
     assert call(op=7) == capi.ERROR_NOT_SUPPORTED
     assert call(kind=5) == capi.ERROR_NOT_SUPPORTED
@@ -129,7 +138,7 @@ def test_reduce_argument_validation():
     assert call(n_out=0) == capi.ERROR_NULL_VIEW
     assert call(n=1 << 31) == capi.ERROR_NOT_SUPPORTED
     assert call(t=capi.I16) == capi.ERROR_NOT_SUPPORTED
-    assert call(stride=3) == capi.ERROR_NOT_SUPPORTED
+    assert call(stride=0) == capi.ERROR_OUT_OF_RANGE
     assert call(tb=16) == capi.ERROR_OUT_OF_RANGE
 
 
@@ -148,7 +157,7 @@ def test_histogram_argument_validation():
     assert call(t=capi.F16) == capi.ERROR_NOT_SUPPORTED
     assert call(bt=capi.F32) == capi.ERROR_NOT_SUPPORTED
     assert call(loc=9) == capi.ERROR_NOT_SUPPORTED
-    assert call(stride=2) == capi.ERROR_NOT_SUPPORTED
+    assert call(stride=0) == capi.ERROR_OUT_OF_RANGE
 
 
 def test_missing_library_fails_loudly(monkeypatch):

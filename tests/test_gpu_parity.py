@@ -462,3 +462,135 @@ def test_sort_reuses_dirty_temp_and_unaligned_key_view():
     out = d.numpy()
     assert np.array_equal(out[3:50003], np.sort(keys[3:50003]))
     assert np.array_equal(out[:3], keys[:3]) and np.array_equal(out[50003:], keys[50003:])
+
+
+# ------------------------------------------------------ strided views (General)
+# Stride1D.General with an element stride above one (ArrayViews.tt:114-119):
+# element i of the view is base[i * stride].  The logical elements must match
+# the oracle on the dense sequence, and the elements in between must be left
+# exactly as they were.
+SENTINEL = 0x5A
+
+
+def strided_buffer(logical: np.ndarray, stride: int):
+    """A physical buffer holding `logical` at multiples of `stride`, sentinel
+    bytes elsewhere; returns (device array, strided view, host copy)."""
+    phys = np.full(((logical.size - 1) * stride + 1) * logical.dtype.itemsize,
+                   SENTINEL, dtype=np.uint8).view(logical.dtype).copy()
+    phys[::stride] = logical
+    dev = D.from_numpy(phys)
+    return dev, dev.strided(stride), phys
+
+
+def assert_gaps_untouched(after: np.ndarray, before: np.ndarray, stride: int):
+    mask = np.ones(after.size, dtype=bool)
+    mask[::stride] = False
+    assert np.array_equal(after.view(np.uint8).reshape(after.size, -1)[mask],
+                          before.view(np.uint8).reshape(before.size, -1)[mask])
+
+
+@pytest.mark.parametrize("stride", [2, 3, 7])
+@pytest.mark.parametrize("dtype", [np.uint32, np.int64, np.float32, np.uint8])
+def test_sort_keys_strided(dtype, stride):
+    for n in [1, 33, 1027, 50001]:
+        note("sort strided", np.dtype(dtype).name, stride, n)
+        keys = (random_float_bits(dtype, n, seed=n) if np.dtype(dtype).kind == "f"
+                else random_ints(dtype, n, seed=n))
+        dev, view, phys = strided_buffer(keys, stride)
+        capi.radix_sort_keys(view)
+        sync()
+        out = dev.numpy()
+        expect = O.radix_sort(keys)
+        assert np.array_equal(np.ascontiguousarray(out[::stride]).view(np.uint8),
+                              expect.view(np.uint8))
+        assert_gaps_untouched(out, phys, stride)
+
+
+@pytest.mark.parametrize("key_stride,value_stride", [(2, 1), (1, 3), (4, 5)])
+def test_sort_pairs_strided(key_stride, value_stride):
+    for n in [1, 127, 40000]:
+        note("pairs strided", key_stride, value_stride, n)
+        keys = random_ints(np.uint16, n, seed=n)        # many duplicates
+        vals = np.arange(n, dtype=np.uint64) * 3 + 1
+        kdev, kview, kphys = strided_buffer(keys, key_stride)
+        vdev, vview, vphys = strided_buffer(vals, value_stride)
+        capi.radix_sort_pairs(kview, vview)
+        sync()
+        ek, ev = O.radix_sort_pairs(keys, vals)
+        kout, vout = kdev.numpy(), vdev.numpy()
+        assert np.array_equal(kout[::key_stride], ek)
+        assert np.array_equal(vout[::value_stride], ev)
+        assert_gaps_untouched(kout, kphys, key_stride)
+        assert_gaps_untouched(vout, vphys, value_stride)
+        # sequencer form: values = stable permutation indices
+        kdev, kview, _ = strided_buffer(keys, key_stride)
+        idev, iview, iphys = strided_buffer(np.zeros(n, dtype=np.int32), value_stride)
+        capi.radix_sort_pairs(kview, iview, values_from_index=True)
+        sync()
+        order = np.argsort(keys, kind="stable").astype(np.int32)
+        iout = idev.numpy()
+        assert np.array_equal(iout[::value_stride], order)
+        assert_gaps_untouched(iout, iphys, value_stride)
+
+
+@pytest.mark.parametrize("in_stride,out_stride", [(2, 1), (1, 2), (3, 5), (4, 4)])
+@pytest.mark.parametrize("dtype", [np.int32, np.uint64, np.float64])
+def test_scan_strided(dtype, in_stride, out_stride):
+    for n in [1, 31, 1027, 70001]:
+        for kind in (capi.SCAN_INCLUSIVE, capi.SCAN_EXCLUSIVE):
+            for op in OPS:
+                note("scan strided", np.dtype(dtype).name, in_stride, out_stride, n, kind, op)
+                v = (random_ints(dtype, n, seed=n, lo=0, hi=1000)
+                     if np.dtype(dtype).kind in "iu"
+                     else np.random.default_rng(n).integers(-50, 50, n).astype(dtype))
+                idev, iview, iphys = strided_buffer(v, in_stride)
+                odev, oview, ophys = strided_buffer(np.zeros(n, dtype=dtype), out_stride)
+                capi.scan(iview, oview, op=op, kind=kind)
+                sync()
+                expect = O.scan(v, op=op, inclusive=kind == capi.SCAN_INCLUSIVE)
+                out = odev.numpy()
+                assert np.array_equal(out[::out_stride], expect)
+                assert_gaps_untouched(out, ophys, out_stride)
+                assert np.array_equal(idev.numpy().view(np.uint8), iphys.view(np.uint8))
+
+
+def test_scan_strided_in_place():
+    v = random_ints(np.int32, 5000, seed=5, lo=-9, hi=9)
+    dev, view, phys = strided_buffer(v, 3)
+    capi.scan(view, view, kind=capi.SCAN_INCLUSIVE)
+    sync()
+    out = dev.numpy()
+    assert np.array_equal(out[::3], O.scan(v, op=capi.OP_ADD, inclusive=True))
+    assert_gaps_untouched(out, phys, 3)
+
+
+@pytest.mark.parametrize("stride", [2, 5])
+@pytest.mark.parametrize("dtype", [np.int32, np.uint64, np.float32])
+def test_reduce_strided(dtype, stride):
+    for n in [1, 63, 4097, 300001]:
+        for op in OPS:
+            note("reduce strided", np.dtype(dtype).name, stride, n, op)
+            v = (random_ints(dtype, n, seed=n) if np.dtype(dtype).kind in "iu"
+                 else np.random.default_rng(n).integers(-10, 10, n).astype(dtype))
+            dev, view, _ = strided_buffer(v, stride)
+            out = D.zeros(1, dtype)
+            capi.reduce(view, out, op=op)
+            sync()
+            assert out.numpy()[0] == O.reduce(v, op=op)
+
+
+@pytest.mark.parametrize("stride", [2, 9])
+@pytest.mark.parametrize("num_bins", [64, 256, 20000])
+def test_histogram_strided(num_bins, stride):
+    for n in [1, 1024, 200003]:
+        note("histogram strided", num_bins, stride, n)
+        v = random_ints(np.int32, n, seed=n, lo=-5, hi=3 * num_bins)
+        dev, view, _ = strided_buffer(v, stride)
+        bins = D.zeros(num_bins, np.int32)
+        ov = D.zeros(1, np.int32)
+        capi.histogram(view, bins, ov, locator=capi.LOCATOR_MODULO)
+        sync()
+        eb, eo = O.histogram(v, np.zeros(num_bins, np.int32),
+                             locator=O.LOCATOR_MODULO)
+        assert np.array_equal(bins.numpy(), eb)
+        assert ov.numpy()[0] == eo
