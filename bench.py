@@ -370,6 +370,43 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
                      "verified": ok}
         log(f"[bench] {name}: {t:.3f} ms/step, {out[name]['gkeys_per_s']} Gkeys/s")
         del work, keys, temp, o64, src
+
+    # The neighbours of sort and scan in user pipelines.
+    # Unique on sorted Zipf keys (the sort -> unique pipeline): reads n keys,
+    # writes the kept ones.
+    src = torch.sort(datagen.zipf_u32_torch(n28).to(torch.int64) & 0xFFFFFFFF)[0].to(torch.int32)
+    work = torch.empty_like(src)
+    d, count = wrap(work, np.uint32), D.zeros(1, np.int64)
+    temp = capi.temp_buffer(capi.unique_temp_bytes(n28, np.uint32))
+    distinct = int(torch.unique_consecutive(src).numel())
+    e = timed("unique_u32_sorted_zipf_2^28", lambda: work.copy_(src),
+              lambda: capi.unique(d, count, temp), 4.0 * (n28 + distinct), "unique")
+    kept = int(count.numpy()[0])
+    e["kept"] = kept
+    e["verified"] = kept == distinct and bool(
+        (work[:kept] == torch.unique_consecutive(src)).all().item())
+    # all-distinct input: every element is written back
+    seq = torch.arange(n28, dtype=torch.int32, device="cuda:0")
+    e = timed("unique_i32_all_distinct_2^28", lambda: work.copy_(seq),
+              lambda: capi.unique(d, count, temp), 8.0 * n28, "unique")
+    e["verified"] = int(count.numpy()[0]) == n28 and bool((work == seq).all().item())
+    del src, seq, temp
+
+    # Sequence (iota) and Initialize (fill) of 2^28 int32: n * 4 bytes written.
+    d = wrap(work, np.int32)
+    e = timed("sequence_i32_2^28", nothing, lambda: capi.sequence(d), 4.0 * n28, "sequence")
+    e["verified"] = bool((work == torch.arange(n28, dtype=torch.int32, device="cuda:0")).all().item())
+    e = timed("initialize_i32_2^28", nothing, lambda: capi.initialize(d, 7), 4.0 * n28,
+              "initialize")
+    e["verified"] = bool((work == 7).all().item())
+    # Reorder by a random permutation: a gather, n * (4 + 4 + 4) bytes.
+    perm = torch.randperm(n28, device="cuda:0", generator=torch.Generator("cuda:0").manual_seed(1)).to(torch.int32)
+    source = datagen.uniform_u32_torch(n28)
+    e = timed("reorder_u32_random_permutation_2^28", nothing,
+              lambda: capi.reorder(wrap(source, np.uint32), d, wrap(perm, np.int32)),
+              12.0 * n28, "reorder")
+    e["verified"] = bool((work == source[perm.to(torch.int64)]).all().item())
+    del work, perm, source
     return out
 
 

@@ -44,6 +44,8 @@ EXPORTS = [
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
+    "ilgpu_hip_unique_temp_bytes", "ilgpu_hip_unique", "ilgpu_hip_initialize",
+    "ilgpu_hip_sequence", "ilgpu_hip_reorder",
 ]
 
 _NP_TO_TYPE = {
@@ -127,6 +129,11 @@ def lib() -> ctypes.CDLL:
         L.ilgpu_hip_scan.argtypes = [vp, vp, i64, i64, vp, i64, i64, i32, i32,
                                      i32, vp, i64]
         L.ilgpu_hip_reduce_temp_bytes.argtypes = [i64, i32, p64]
+        L.ilgpu_hip_unique_temp_bytes.argtypes = [i64, i32, p64]
+        L.ilgpu_hip_unique.argtypes = [vp, vp, i64, i32, vp, i64, vp, i64]
+        L.ilgpu_hip_initialize.argtypes = [vp, vp, i64, i64, i32, vp]
+        L.ilgpu_hip_sequence.argtypes = [vp, vp, i64, i64, i32, i64, i64]
+        L.ilgpu_hip_reorder.argtypes = [vp, vp, i64, vp, i64, vp, i64, i32]
         L.ilgpu_hip_reduce.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64, vp, i64]
         L.ilgpu_hip_histogram.argtypes = [vp, vp, i64, i64, i32, vp, i64, i32,
                                           i32, vp]
@@ -324,3 +331,42 @@ def histogram(inp: DeviceArray, bins: DeviceArray,
         bins.ptr,
         bins.length, bins.type_code, locator,
         overflow.ptr if overflow is not None else None))
+
+
+def unique_temp_bytes(n: int, dtype) -> int:
+    return _query(lib().ilgpu_hip_unique_temp_bytes, n, type_code(dtype))
+
+
+def unique(data: DeviceArray, new_length: DeviceArray,
+           temp: Optional[DeviceArray] = None, *, stream=None) -> None:
+    """Removes consecutive duplicates in place; new_length[0] (int64, on the
+    device) receives the number of elements kept."""
+    if temp is None:
+        temp = temp_buffer(unique_temp_bytes(max(data.length, 1), data.dtype))
+    check(lib().ilgpu_hip_unique(
+        _stream_ptr(stream), data.ptr, data.length, data.type_code,
+        new_length.ptr, new_length.length, temp.ptr, temp.nbytes))
+
+
+def initialize(view: DeviceArray, value, *, stream=None) -> None:
+    v = np.ascontiguousarray(np.asarray(value, dtype=view.dtype)).reshape(1)
+    check(lib().ilgpu_hip_initialize(
+        _stream_ptr(stream), view.ptr, view.length, view.stride,
+        view.dtype.itemsize, v.ctypes.data_as(ctypes.c_void_p)))
+
+
+def sequence(view: DeviceArray, *, sequence_length: Optional[int] = None,
+             batch_length: int = 1, stream=None) -> None:
+    """Sequence / RepeatedSequence / BatchedSequence / RepeatedBatchedSequence
+    with the identity sequencer of the view's element type."""
+    check(lib().ilgpu_hip_sequence(
+        _stream_ptr(stream), view.ptr, view.length, view.stride, view.type_code,
+        view.length if sequence_length is None else sequence_length,
+        batch_length))
+
+
+def reorder(source: DeviceArray, target: DeviceArray, order: DeviceArray, *,
+            stream=None) -> None:
+    check(lib().ilgpu_hip_reorder(
+        _stream_ptr(stream), source.ptr, source.length, target.ptr,
+        target.length, order.ptr, order.length, source.dtype.itemsize))

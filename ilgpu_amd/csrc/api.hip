@@ -354,4 +354,88 @@ int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void* in,
                           in_type, bins, num_bins, bin_type, locator, overflow);
 }
 
+/* ---- unique ------------------------------------------------------------ */
+
+int32_t ilgpu_hip_unique_temp_bytes(int64_t n, int32_t elem_type,
+                                    int64_t* temp_bytes) {
+  if (temp_bytes == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  const int eb = elem_size(elem_type);
+  if (eb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (n < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (n > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  *temp_bytes = unique_temp_bytes(n, eb);
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t ilgpu_hip_unique(ilgpu_hip_stream_t stream, void* input, int64_t n,
+                         int32_t elem_type, int64_t* new_length,
+                         int64_t new_length_extent, void* temp,
+                         int64_t temp_bytes) {
+  /* Order of checks as in UniqueExtensions.cs:160-178. */
+  const int eb = elem_size(elem_type);
+  if (eb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(input, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(new_length, new_length_extent)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (temp == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (n > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!aligned_to(input, eb) || !aligned_to(new_length, 8))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int32_t rc = check_temp(temp, temp_bytes, unique_temp_bytes(n, eb));
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  return launch_unique(static_cast<hipStream_t>(stream), input, n, elem_type,
+                       new_length, temp);
+}
+
+/* ---- initialize, sequence, reorder -------------------------------------- */
+
+int32_t ilgpu_hip_initialize(ilgpu_hip_stream_t stream, void* view, int64_t n,
+                             int64_t stride, int32_t elem_bytes,
+                             const void* value) {
+  /* InitializeExtensions.cs:124-127. */
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 &&
+      elem_bytes != 8 && elem_bytes != 16)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(view, n) || value == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(view, elem_bytes)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  return launch_initialize(static_cast<hipStream_t>(stream), view, n, stride,
+                           elem_bytes, value);
+}
+
+int32_t ilgpu_hip_sequence(ilgpu_hip_stream_t stream, void* view, int64_t n,
+                           int64_t stride, int32_t elem_type,
+                           int64_t sequence_length, int64_t batch_length) {
+  /* SequenceExtensions.cs:362-371. */
+  const int eb = elem_size(elem_type);
+  if (eb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(view, n)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (sequence_length < 1 || batch_length < 1 || stride < 1)
+    return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(view, eb)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  return launch_sequence(static_cast<hipStream_t>(stream), view, n, stride,
+                         elem_type, sequence_length, batch_length);
+}
+
+int32_t ilgpu_hip_reorder(ilgpu_hip_stream_t stream, const void* source,
+                          int64_t source_length, void* target,
+                          int64_t target_length, const int32_t* order,
+                          int64_t order_length, int32_t elem_bytes) {
+  /* ReorderExtensions.cs:158-171, then TransformExtensions.cs:318-332 with the
+   * order view as the transformer's source. */
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 &&
+      elem_bytes != 8 && elem_bytes != 16)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(source, source_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(order, order_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (order_length < source_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (source_length > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(target, target_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (target_length < order_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(source, elem_bytes) || !aligned_to(target, elem_bytes) ||
+      !aligned_to(order, 4))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  return launch_reorder(static_cast<hipStream_t>(stream), source, target, order,
+                        order_length, elem_bytes);
+}
+
 }  // extern "C"

@@ -45,6 +45,20 @@ int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
 int64_t radix_sort_max_length();
 int32_t launch_radix_sort(hipStream_t stream, const SortArgs& args);
 
+// scan.hip: Unique (consecutive duplicates removed in place, new length to
+// out_length[0] on the device).
+int64_t unique_temp_bytes(int64_t n, int elem_bytes);
+int32_t launch_unique(hipStream_t stream, void* data, int64_t n, int32_t type,
+                      int64_t* out_length, void* temp);
+
+// sequence.hip
+int32_t launch_initialize(hipStream_t stream, void* view, int64_t n, int64_t stride,
+                          int elem_bytes, const void* value);
+int32_t launch_sequence(hipStream_t stream, void* view, int64_t n, int64_t stride,
+                        int32_t type, int64_t sequence_length, int64_t batch_length);
+int32_t launch_reorder(hipStream_t stream, const void* source, void* target,
+                       const int32_t* order, int64_t n, int elem_bytes);
+
 // fill kernel shared by scan and sort: words[0..count) = 0, as a kernel so
 // that callers may capture the stream into a graph.
 int32_t launch_zero_words(hipStream_t stream, uint32_t* words, int64_t count);

@@ -271,6 +271,146 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
   }
 }
 
+// ---- unique ------------------------------------------------------------------
+// Removes consecutive duplicates in place and reports the new length; stands
+// in for the Unique delegate of UniqueExtensions.cs:59-209, whose kernel runs
+// the groups strictly one after the other (SequentialGroupExecutor) with a
+// serial compaction loop per group.  Here it is the same single-pass chain as
+// the scan: an element is kept if it differs from its predecessor, a tile
+// publishes its number of kept elements, resolves how many were kept in front
+// of it, and writes its kept elements to data[kept_before + local rank].
+//
+// In place is safe without a second buffer: a tile loads all of its elements
+// (and the element in front of each vector) before it publishes anything, a
+// tile learns its offset only after every earlier tile has published, and it
+// writes only at or below the positions it read, so no element is overwritten
+// before its owner (or its successor's comparison) has read it.
+//
+// "Differs" is Comparison<T>.Compare(a, b) != 0 (ComparisonOperations.tt:30-45),
+// i.e. CompareTo: all NaNs are equal to each other and -0.0 equals +0.0.
+#ifndef ILGPU_HIP_UNIQUE_VECS
+#define ILGPU_HIP_UNIQUE_VECS 8
+#endif
+constexpr int kUniqueVecs = ILGPU_HIP_UNIQUE_VECS;
+
+template <typename T> struct is_float_like { static constexpr bool value = is_fp<T>::value; };
+template <> struct is_float_like<_Float16> { static constexpr bool value = true; };
+
+template <typename T> __device__ __forceinline__ bool differs(T a, T b) {
+  if constexpr (is_float_like<T>::value) return !(a == b) && !(a != a && b != b);
+  else return a != b;
+}
+
+template <typename T> constexpr int unique_tile_elems() {
+  return kBlock * kUniqueVecs * Vec16<T>::N;
+}
+
+template <typename T, bool VECTOR>
+__global__ __launch_bounds__(kBlock) void unique_kernel(
+    T* data, int64_t n, int64_t* __restrict__ out_length,
+    uint32_t* __restrict__ ticket, TileState<uint32_t> st, int num_tiles) {
+  using V = typename Vec16<T>::type;
+  constexpr int VN = Vec16<T>::N;
+  constexpr int kTile = unique_tile_elems<T>();
+  constexpr int kWaveElems = kTile / kWaves;
+
+  __shared__ int s_tile;
+  __shared__ uint32_t s_wave_total[kWaves];
+  __shared__ uint32_t s_prefix;
+
+  if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
+  __syncthreads();
+  const int tile = s_tile;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  const int64_t tile_base = (int64_t)tile * kTile;
+  const int64_t wave_base = tile_base + (int64_t)wave * kWaveElems;
+  const bool full = tile_base + kTile <= n;
+
+  T x[kUniqueVecs][VN];
+  // The element in front of the wave's chunk; every other predecessor is in a
+  // register of this wave.
+  const T chunk_before = wave_base > 0 && wave_base < n ? data[wave_base - 1] : T();
+#pragma unroll
+  for (int j = 0; j < kUniqueVecs; ++j) {
+    const int64_t first = wave_base + (int64_t)(j * kWaveSize + lane) * VN;
+    if (VECTOR && full) {
+      const V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(data + first));
+#pragma unroll
+      for (int k = 0; k < VN; ++k) x[j][k] = v[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) x[j][k] = first + k < n ? data[first + k] : T();
+    }
+  }
+  T before[kUniqueVecs];  // the element in front of each vector
+#pragma unroll
+  for (int j = 0; j < kUniqueVecs; ++j) {
+    const T from_left = shfl_up(x[j][VN - 1], 1);
+    const T row_before = j == 0 ? chunk_before : shfl(x[j > 0 ? j - 1 : 0][VN - 1], kWaveSize - 1);
+    before[j] = lane == 0 ? row_before : from_left;
+  }
+
+  // keep bit k of vector j; kept elements per vector; wave scan per row.
+  uint32_t keep[kUniqueVecs], lane_excl[kUniqueVecs], seg_total[kUniqueVecs];
+#pragma unroll
+  for (int j = 0; j < kUniqueVecs; ++j) {
+    const int64_t first = wave_base + (int64_t)(j * kWaveSize + lane) * VN;
+    uint32_t bits = 0;
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      const bool valid = first + k < n;
+      const bool is_first = first + k == 0;
+      const bool d = differs<T>(x[j][k], k == 0 ? before[j] : x[j][k - 1]);
+      if (valid && (is_first || d)) bits |= 1u << k;
+    }
+    keep[j] = bits;
+    const uint32_t cnt = (uint32_t)__popc(bits);
+    const uint32_t inc = wave_inclusive_scan<uint32_t, ILGPU_HIP_OP_ADD>(cnt, lane);
+    seg_total[j] = shfl(inc, kWaveSize - 1);
+    lane_excl[j] = inc - cnt;
+  }
+  uint32_t wave_total = 0;
+#pragma unroll
+  for (int j = 0; j < kUniqueVecs; ++j) wave_total += seg_total[j];
+  if (lane == 0) s_wave_total[wave] = wave_total;
+  __syncthreads();
+
+  uint32_t wave_prefix = 0, block_total = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    if (w == wave) wave_prefix = block_total;
+    block_total += s_wave_total[w];
+  }
+  if (wave == 0) {
+    const uint32_t exclusive =
+        resolve_prefix<uint32_t, ILGPU_HIP_OP_ADD>(st, tile, block_total, lane);
+    if (lane == 0) s_prefix = exclusive;
+  }
+  __syncthreads();
+
+  uint32_t running = s_prefix + wave_prefix;
+#pragma unroll
+  for (int j = 0; j < kUniqueVecs; ++j) {
+    uint32_t pos = running + lane_excl[j];
+    if (keep[j] == (1u << VN) - 1u) {
+      // the whole vector survives: one 16-byte store, aligned like an element
+      typedef V UnalignedV __attribute__((aligned(sizeof(T))));
+      V v;
+#pragma unroll
+      for (int k = 0; k < VN; ++k) v[k] = x[j][k];
+      *reinterpret_cast<UnalignedV*>(data + pos) = v;
+    } else {
+#pragma unroll
+      for (int k = 0; k < VN; ++k)
+        if (keep[j] >> k & 1u) data[pos++] = x[j][k];
+    }
+    running += seg_total[j];
+  }
+  if (tile == num_tiles - 1 && threadIdx.x == 0)
+    out_length[0] = (int64_t)s_prefix + (int64_t)block_total;
+}
+
 __global__ void zero_words_kernel(uint32_t* words, int64_t count) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count;
@@ -377,6 +517,56 @@ int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
     case ILGPU_HIP_U64: return launch_op<uint64_t>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
     case ILGPU_HIP_F32: return launch_op<float>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
     case ILGPU_HIP_F64: return launch_op<double>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
+    default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  }
+}
+
+int64_t unique_temp_bytes(int64_t n, int elem_bytes) {
+  const int64_t tile = (int64_t)kBlock * kUniqueVecs * (16 / elem_bytes);
+  return 256 + kHeaderBytes + div_up(n, tile) * 8;
+}
+
+namespace {
+template <typename T>
+int32_t launch_unique_typed(hipStream_t stream, void* data, int64_t n,
+                            int64_t* out_length, void* temp) {
+  const int64_t tiles = div_up(n, (int64_t)unique_tile_elems<T>());
+  char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)temp, 256));
+  uint32_t* ticket = reinterpret_cast<uint32_t*>(base);
+  TileState<uint32_t> st;
+  st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
+  const int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
+                                       (kHeaderBytes + tiles * 8) / 4);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  const bool vector = (reinterpret_cast<uintptr_t>(data) & 15) == 0;
+  ProfileScope scope(stream, "unique");
+  if (vector)
+    hipLaunchKernelGGL((unique_kernel<T, true>), dim3((unsigned)tiles), dim3(kBlock), 0,
+                       stream, static_cast<T*>(data), n, out_length, ticket, st,
+                       (int)tiles);
+  else
+    hipLaunchKernelGGL((unique_kernel<T, false>), dim3((unsigned)tiles), dim3(kBlock), 0,
+                       stream, static_cast<T*>(data), n, out_length, ticket, st,
+                       (int)tiles);
+  ILGPU_HIP_CHECK(hipGetLastError());
+  return ILGPU_HIP_SUCCESS;
+}
+}  // namespace
+
+int32_t launch_unique(hipStream_t stream, void* data, int64_t n, int32_t type,
+                      int64_t* out_length, void* temp) {
+  switch (type) {
+    case ILGPU_HIP_I8: return launch_unique_typed<int8_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_U8: return launch_unique_typed<uint8_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_I16: return launch_unique_typed<int16_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_U16: return launch_unique_typed<uint16_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_I32: return launch_unique_typed<int32_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_U32: return launch_unique_typed<uint32_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_I64: return launch_unique_typed<int64_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_U64: return launch_unique_typed<uint64_t>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_F16: return launch_unique_typed<_Float16>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_F32: return launch_unique_typed<float>(stream, data, n, out_length, temp);
+    case ILGPU_HIP_F64: return launch_unique_typed<double>(stream, data, n, out_length, temp);
     default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
 }

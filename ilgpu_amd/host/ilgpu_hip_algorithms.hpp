@@ -282,7 +282,24 @@ using Int32Sequencer = IndexValueSequencer<int32_t>;
 using Int64Sequencer = IndexValueSequencer<int64_t>;
 using UInt32Sequencer = IndexValueSequencer<uint32_t>;
 using UInt64Sequencer = IndexValueSequencer<uint64_t>;
+using Int8Sequencer = IndexValueSequencer<int8_t>;
+using Int16Sequencer = IndexValueSequencer<int16_t>;
+using UInt8Sequencer = IndexValueSequencer<uint8_t>;
+using UInt16Sequencer = IndexValueSequencer<uint16_t>;
+using FloatSequencer = IndexValueSequencer<float>;
+using DoubleSequencer = IndexValueSequencer<double>;
 }  // namespace Sequencers
+
+// Comparison<T> (ComparisonOperations.tt:30-45): CompareTo.
+namespace ComparisonOperations {
+template <typename T> struct Comparison { using Type = T; };
+using ComparisonInt8 = Comparison<int8_t>;     using ComparisonInt16 = Comparison<int16_t>;
+using ComparisonInt32 = Comparison<int32_t>;   using ComparisonInt64 = Comparison<int64_t>;
+using ComparisonUInt8 = Comparison<uint8_t>;   using ComparisonUInt16 = Comparison<uint16_t>;
+using ComparisonUInt32 = Comparison<uint32_t>; using ComparisonUInt64 = Comparison<uint64_t>;
+using ComparisonHalf = Comparison<Half>;       using ComparisonFloat = Comparison<float>;
+using ComparisonDouble = Comparison<double>;
+}  // namespace ComparisonOperations
 
 namespace Algorithms {
 
@@ -661,6 +678,154 @@ template <typename T, typename TStride, typename TLocator, typename TBinType>
 void HistogramUnchecked(Accelerator& accelerator, AcceleratorStream& stream,
                         ArrayView1D<T, TStride> view, ArrayView<TBinType> histogram) {
   CreateHistogramUnchecked<T, TStride, TBinType, TLocator>(accelerator)(stream, view, histogram);
+}
+
+// ---- unique (UniqueExtensions.cs) ------------------------------------------------
+template <typename T>
+using UniqueDelegate = std::function<void(AcceleratorStream&, ArrayView<T>, ArrayView<int64_t>,
+                                          ArrayView<int32_t>)>;
+// ComputeUniqueTempStorageSize (:116-123), in 32-bit ints.
+template <typename T>
+int64_t ComputeUniqueTempStorageSize(Accelerator&, int64_t dataLength) {
+  int64_t bytes = 0;
+  HipAlgorithmsException::ThrowIfFailed(
+      ilgpu_hip_unique_temp_bytes(dataLength, TypeCode<T>::value, &bytes), "dataLength");
+  return (bytes + 3) / 4;
+}
+// CreateUnique (:133-190).
+template <typename T, typename TComparisonOperation>
+UniqueDelegate<T> CreateUnique(Accelerator& accelerator) {
+  static_assert(std::is_same<typename TComparisonOperation::Type, T>::value,
+                "comparison operation and element type differ");
+  Accelerator* accl = &accelerator;
+  return [accl](AcceleratorStream& stream, ArrayView<T> input, ArrayView<int64_t> output,
+                ArrayView<int32_t> temp) {
+    if (!input.IsValid()) throw ArgumentNullException("input");
+    if (!output.IsValid()) throw ArgumentNullException("output");
+    if (!temp.IsValid()) throw ArgumentNullException("temp");
+    if (output.Length() < 1) throw ArgumentOutOfRangeException("output");
+    if (input.Length() > std::numeric_limits<int32_t>::max())
+      throw NotSupportedException("NotSupportedArrayView64");
+    if (temp.Length() < ComputeUniqueTempStorageSize<T>(*accl, input.Length()))
+      throw ArgumentOutOfRangeException("temp");
+    HipAlgorithmsException::ThrowIfFailed(
+        ilgpu_hip_unique(stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(),
+                         TypeCode<T>::value, output.LoadEffectiveAddressAsPtr(), output.Length(),
+                         temp.LoadEffectiveAddressAsPtr(), temp.Length() * 4),
+        "temp");
+  };
+}
+// Unique returning the new length (:199-209): allocates its output and temp and
+// synchronises the stream.
+template <typename T, typename TComparisonOperation>
+int64_t Unique(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<T> input) {
+  auto output = accelerator.Allocate1D<int64_t>(1);
+  auto temp = accelerator.Allocate1D<int32_t>(
+      ComputeUniqueTempStorageSize<T>(accelerator, input.Length()));
+  CreateUnique<T, TComparisonOperation>(accelerator)(stream, input, output->View(),
+                                                     temp->View());
+  stream.Synchronize();
+  return output->GetAsArray1D()[0];
+}
+
+// ---- initialize (InitializeExtensions.cs:116-176) -----------------------------------
+template <typename T, typename TStride>
+using Initializer = std::function<void(AcceleratorStream&, ArrayView1D<T, TStride>, T)>;
+template <typename T, typename TStride>
+Initializer<T, TStride> CreateInitializer(Accelerator&) {
+  static_assert(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8 ||
+                    sizeof(T) == 16,
+                "element sizes of 1, 2, 4, 8 or 16 bytes");
+  return [](AcceleratorStream& stream, ArrayView1D<T, TStride> view, T value) {
+    if (!view.IsValid()) throw ArgumentNullException("view");
+    if (view.Length() < 1) throw ArgumentOutOfRangeException("view");
+    HipAlgorithmsException::ThrowIfFailed(
+        ilgpu_hip_initialize(stream.StreamPtr(), view.LoadEffectiveAddressAsPtr(), view.Length(),
+                             view.Stride().Stride(), (int32_t)sizeof(T), &value),
+        "view");
+  };
+}
+template <typename T>
+void Initialize(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<T> view, T value) {
+  CreateInitializer<T, Stride1D::Dense>(accelerator)(stream, ArrayView1D<T, Stride1D::Dense>(view),
+                                                     value);
+}
+template <typename T, typename TStride>
+void Initialize(Accelerator& accelerator, AcceleratorStream& stream,
+                ArrayView1D<T, TStride> view, T value) {
+  CreateInitializer<T, TStride>(accelerator)(stream, view, value);
+}
+
+// ---- sequence (SequenceExtensions.cs:238-630), identity sequencers -----------------------
+namespace detail {
+template <typename T, typename TStride, typename TSequencer>
+void RunSequencer(AcceleratorStream& stream, ArrayView1D<T, TStride> view,
+                  int64_t sequenceLength, int64_t sequenceBatchLength) {
+  static_assert(std::is_same<typename TSequencer::Type, T>::value,
+                "sequencer and element type differ");
+  HipAlgorithmsException::ThrowIfFailed(
+      ilgpu_hip_sequence(stream.StreamPtr(), view.LoadEffectiveAddressAsPtr(), view.Length(),
+                         view.Stride().Stride(), TypeCode<T>::value, sequenceLength,
+                         sequenceBatchLength),
+      "view");
+}
+template <typename TView> void CheckSequenceView(const TView& view) {
+  if (!view.IsValid()) throw ArgumentNullException("view");
+  if (view.Length() < 1) throw ArgumentOutOfRangeException("view");
+}
+}  // namespace detail
+// Sequence (:513-524): view[i] = sequencer(i).
+template <typename T, typename TStride, typename TSequencer>
+void Sequence(Accelerator&, AcceleratorStream& stream, ArrayView1D<T, TStride> view, TSequencer) {
+  detail::CheckSequenceView(view);
+  detail::RunSequencer<T, TStride, TSequencer>(stream, view, view.Length(), 1);
+}
+// RepeatedSequence (:542-555): view[i] = sequencer(i % sequenceLength).
+template <typename T, typename TStride, typename TSequencer>
+void RepeatedSequence(Accelerator&, AcceleratorStream& stream, ArrayView1D<T, TStride> view,
+                      int64_t sequenceLength, TSequencer) {
+  detail::CheckSequenceView(view);
+  if (sequenceLength < 1) throw ArgumentOutOfRangeException("sequenceLength");
+  detail::RunSequencer<T, TStride, TSequencer>(stream, view, sequenceLength, 1);
+}
+// BatchedSequence (:573-586): view[i] = sequencer(i / sequenceBatchLength).
+template <typename T, typename TStride, typename TSequencer>
+void BatchedSequence(Accelerator&, AcceleratorStream& stream, ArrayView1D<T, TStride> view,
+                     int64_t sequenceBatchLength, TSequencer) {
+  detail::CheckSequenceView(view);
+  if (sequenceBatchLength < 1) throw ArgumentOutOfRangeException("sequenceBatchLength");
+  detail::RunSequencer<T, TStride, TSequencer>(stream, view, view.Length(), sequenceBatchLength);
+}
+// RepeatedBatchedSequence (:613-630).
+template <typename T, typename TStride, typename TSequencer>
+void RepeatedBatchedSequence(Accelerator&, AcceleratorStream& stream,
+                             ArrayView1D<T, TStride> view, int64_t sequenceLength,
+                             int64_t sequenceBatchLength, TSequencer) {
+  detail::CheckSequenceView(view);
+  if (sequenceLength < 1) throw ArgumentOutOfRangeException("sequenceLength");
+  if (sequenceBatchLength < 1) throw ArgumentOutOfRangeException("sequenceBatchLength");
+  detail::RunSequencer<T, TStride, TSequencer>(stream, view, sequenceLength,
+                                               sequenceBatchLength);
+}
+
+// ---- reorder (ReorderExtensions.cs:194-214): target[i] = source[reorderView[i]] -------------
+template <typename T>
+void Reorder(Accelerator&, AcceleratorStream& stream, ArrayView<T> source, ArrayView<T> target,
+             ArrayView<Index1D> reorderView) {
+  if (!source.IsValid()) throw ArgumentNullException("source");
+  if (source.Length() < 1) throw ArgumentOutOfRangeException("source");
+  if (!reorderView.IsValid()) throw ArgumentNullException("reorderView");
+  if (reorderView.Length() < source.Length()) throw ArgumentOutOfRangeException("reorderView");
+  if (source.Length() > std::numeric_limits<int32_t>::max())
+    throw NotSupportedException("NotSupportedArrayView64");
+  if (!target.IsValid()) throw ArgumentNullException("source");  // sic, TransformExtensions.cs:322-323
+  if (target.Length() < reorderView.Length()) throw ArgumentOutOfRangeException("target");
+  HipAlgorithmsException::ThrowIfFailed(
+      ilgpu_hip_reorder(stream.StreamPtr(), source.LoadEffectiveAddressAsPtr(), source.Length(),
+                        target.LoadEffectiveAddressAsPtr(), target.Length(),
+                        reorderView.LoadEffectiveAddressAsPtr(), reorderView.Length(),
+                        (int32_t)sizeof(T)),
+      "target");
 }
 
 }  // namespace Algorithms

@@ -214,6 +214,48 @@ int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void *in,
                             void *bins, int64_t num_bins, int32_t bin_type,
                             int32_t locator, int32_t *overflow);
 
+/* ---- unique -------------------------------------------------------------
+ * Replaces: the Unique<T> delegate made by CreateUnique<T, Comparison<T>>, the
+ * value-returning Unique and ComputeUniqueTempStorageSize
+ * (UniqueExtensions.cs:27-33, 116-209).  Removes consecutive duplicates of
+ * input[0..n) in place and writes the new length to new_length[0] (a device
+ * int64, the reference's ArrayView<long> output).  Two elements are duplicates
+ * if Comparison<T>.Compare yields 0 (ComparisonOperations.tt:30-45): CompareTo,
+ * so all NaNs are equal and -0.0 equals +0.0.  elem_type: any of the eleven
+ * numeric types.
+ */
+int32_t ilgpu_hip_unique_temp_bytes(int64_t n, int32_t elem_type,
+                                    int64_t *temp_bytes);
+int32_t ilgpu_hip_unique(ilgpu_hip_stream_t stream, void *input, int64_t n,
+                         int32_t elem_type, int64_t *new_length,
+                         int64_t new_length_extent, void *temp,
+                         int64_t temp_bytes);
+
+/* ---- initialize, sequence, reorder ----------------------------------------
+ * Replace: Initializer delegates and Initialize (InitializeExtensions.cs:26-31,
+ * 116-176): view[i] = *value, `value` being a HOST pointer to elem_bytes bytes
+ * (1, 2, 4, 8 or 16); the Sequencer, RepeatedSequencer, BatchedSequencer and
+ * RepeatedBatchedSequencer delegates (SequenceExtensions.cs:31-123, 238-630)
+ * for the identity sequencers (Sequencers.tt:25-37, IndexSequencer):
+ * view[i] = (T)((i / batch_length) % sequence_length), where Sequence passes
+ * sequence_length = n and batch_length = 1; and Reorder
+ * (ReorderExtensions.cs:194-214): target[i] = source[order[i]] for
+ * i < order_length, with the reference's checks order_length >= source_length
+ * and target_length >= order_length.  Index values are not range-checked.
+ * Transformers with user-written functors are not offered: they need the
+ * reference's JIT.
+ */
+int32_t ilgpu_hip_initialize(ilgpu_hip_stream_t stream, void *view, int64_t n,
+                             int64_t stride, int32_t elem_bytes,
+                             const void *value);
+int32_t ilgpu_hip_sequence(ilgpu_hip_stream_t stream, void *view, int64_t n,
+                           int64_t stride, int32_t elem_type,
+                           int64_t sequence_length, int64_t batch_length);
+int32_t ilgpu_hip_reorder(ilgpu_hip_stream_t stream, const void *source,
+                          int64_t source_length, void *target,
+                          int64_t target_length, const int32_t *order,
+                          int64_t order_length, int32_t elem_bytes);
+
 #ifdef __cplusplus
 }
 #endif

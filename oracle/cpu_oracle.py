@@ -64,6 +64,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_sum_f64.restype = ctypes.c_double
         L.oracle_histogram.argtypes = [i32, i32, i32, vp, i64, vp, i64, vp]
         L.oracle_scan_temp_ints_cpu.restype = i64
+        L.oracle_unique.argtypes = [i32, vp, i64, i64]
+        L.oracle_unique.restype = i64
         L.oracle_radix_sort_temp_ints_cpu.argtypes = [i32, i64, i32]
         L.oracle_radix_sort_temp_ints_cpu.restype = i64
         L.oracle_temp_view_allocate.argtypes = [i64, i64, i32, i32, i64]
@@ -154,6 +156,46 @@ def histogram(values: np.ndarray, bins: np.ndarray,
     if rc != 0:
         raise RuntimeError(f"oracle_histogram failed: {rc}")
     return b, int(ov[0])
+
+
+def unique(values: np.ndarray, tile: int = CPU_GROUP_SIZE) -> np.ndarray:
+    """UniqueExtensions.cs:59-118: the kept prefix after removing consecutive
+    duplicates under Comparison<T> (CompareTo)."""
+    a = np.ascontiguousarray(values).copy()
+    if a.size == 0:
+        return a
+    kept = lib().oracle_unique(type_code(a.dtype), _ptr(a), a.size, tile)
+    if kept < 0:
+        raise RuntimeError("oracle_unique failed")
+    return a[:kept]
+
+
+def sequence(n: int, dtype, sequence_length=None, batch_length: int = 1) -> np.ndarray:
+    """SequenceExtensions.cs:163-171 with the identity sequencers
+    (Sequencers.tt:25-37): view[i] = (T)((i / batchLength) % sequenceLength);
+    Sequence itself passes sequenceLength = view.Length, batchLength = 1
+    (SequenceExtensions.cs:262-268).  The cast is C#'s unchecked conversion
+    from long: wrap-around for integers, nearest value for floating point."""
+    if sequence_length is None:
+        sequence_length = n
+    idx = (np.arange(n, dtype=np.int64) // batch_length) % sequence_length
+    dt = np.dtype(dtype)
+    if dt.kind in "iu":
+        return idx.astype(np.uint64).astype(dt) if dt.kind == "u" else idx.astype(dt)
+    with np.errstate(over="ignore"):   # Half: indices above 65504 become +inf
+        return idx.astype(dt)
+
+
+def initialize(n: int, value) -> np.ndarray:
+    """InitializeExtensions.cs:63-69: view[i] = value."""
+    v = np.asarray(value)
+    return np.full(n, v, dtype=v.dtype)
+
+
+def reorder(source: np.ndarray, order: np.ndarray) -> np.ndarray:
+    """ReorderExtensions.cs:116-120 with IdentityTransformer:
+    target[i] = source[reorderView[i]]."""
+    return np.ascontiguousarray(source)[np.asarray(order, dtype=np.int64)]
 
 
 def scan_temp_ints_cpu() -> int:

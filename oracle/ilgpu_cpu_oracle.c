@@ -555,6 +555,90 @@ int oracle_histogram(int in_type, int bin_type, int locator, const void *in,
   }
 }
 
+/* ----------------------------------------------------------------- unique */
+
+static float half_bits_to_float(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu, bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else {                       /* subnormal: normalise */
+      int e = -1;
+      do { man <<= 1; ++e; } while ((man & 0x400u) == 0);
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7F800000u | (man << 13);
+  } else {
+    bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+/* Comparison<T>.Compare(first, second) = first.CompareTo(second)
+ * (ComparisonOperations.tt:30-45).  .NET CompareTo on floating-point types
+ * orders NaN below everything and equal to NaN; -0.0 equals +0.0. */
+static int compare_to_f64(double a, double b) {
+  if (a < b) return -1;
+  if (a > b) return 1;
+  if (a == b) return 0;
+  if (a != a) return b != b ? 0 : -1;
+  return 1;
+}
+
+static int compare_elements(int type, const char *data, int64_t i, int64_t j) {
+  switch (type) {
+    case ORACLE_I8: { int8_t a = ((const int8_t *)data)[i], b = ((const int8_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_U8: { uint8_t a = ((const uint8_t *)data)[i], b = ((const uint8_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_I16: { int16_t a = ((const int16_t *)data)[i], b = ((const int16_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_U16: { uint16_t a = ((const uint16_t *)data)[i], b = ((const uint16_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_I32: { int32_t a = ((const int32_t *)data)[i], b = ((const int32_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_U32: { uint32_t a = ((const uint32_t *)data)[i], b = ((const uint32_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_I64: { int64_t a = ((const int64_t *)data)[i], b = ((const int64_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_U64: { uint64_t a = ((const uint64_t *)data)[i], b = ((const uint64_t *)data)[j]; return (a > b) - (a < b); }
+    case ORACLE_F16: return compare_to_f64(half_bits_to_float(((const uint16_t *)data)[i]),
+                                           half_bits_to_float(((const uint16_t *)data)[j]));
+    case ORACLE_F32: return compare_to_f64(((const float *)data)[i], ((const float *)data)[j]);
+    default: return compare_to_f64(((const double *)data)[i], ((const double *)data)[j]);
+  }
+}
+
+/* UniqueKernel (UniqueExtensions.cs:59-118) with the groups run one after the
+ * other, as its SequentialGroupExecutor enforces: group g owns elements
+ * [g * tile, (g + 1) * tile); an element is flagged if it differs from its
+ * predecessor, where the first element of a group other than the first is
+ * compared with the last element kept so far (input[output[0] - 1]); thread 0
+ * then compacts the flagged elements to input[output[0]...] in order. */
+int64_t oracle_unique(int type, void *data, int64_t n, int64_t tile) {
+  const int size = oracle_elem_size(type);
+  if (size < 0 || n < 0 || tile < 1) return -1;
+  char *bytes = (char *)data;
+  unsigned char *flags = (unsigned char *)malloc((size_t)tile);
+  if (!flags) return -1;
+  int64_t kept = 0;
+  for (int64_t start = 0; start < n; start += tile) {
+    const int64_t end = start + tile < n ? start + tile : n;
+    for (int64_t i = start; i < end; ++i) {
+      if (i == 0) {
+        flags[0] = 1;
+      } else {
+        const int64_t prev = i == start ? kept - 1 : i - 1;
+        flags[i - start] = compare_elements(type, bytes, i, prev) != 0;
+      }
+    }
+    for (int64_t i = start; i < end; ++i)
+      if (flags[i - start]) {
+        memmove(bytes + kept * size, bytes + i * size, (size_t)size);
+        ++kept;
+      }
+  }
+  free(flags);
+  return kept;
+}
+
 /* ------------------------------------------------------------ temp sizes */
 
 /* ScanExtensions.cs:158-170: AcceleratorType.CPU => 1. */

@@ -22,6 +22,14 @@
  *                               one admissible order of a non-deterministic
  *                               reference (tolerance contract, see oracle_sum_f64).
  *   oracle_histogram            pinned against HistogramTests.tt:50-76 vectors.
+ *   oracle_unique               pinned against RemoveConsecutiveDuplicates on the
+ *                               reference's inputs (UniqueExtensionTests.tt:36-67,
+ *                               integers) and against a first-of-run filter for
+ *                               every tile size; NaN and signed-zero equality follow
+ *                               .NET CompareTo and are pinned by that definition
+ *                               only (no reference test has such inputs).
+ *   sequence / initialize / reorder (numpy restatements in cpu_oracle.py) pinned by
+ *                               SequencerTests.tt:56-70 and ReorderExtensionTests.tt.
  *   temp-size helpers           pinned by the closed formulas they restate.
  */
 #ifndef ILGPU_CPU_ORACLE_H
@@ -89,6 +97,11 @@ double oracle_sum_f64(int type, const void *in, int64_t n);
 int oracle_histogram(int in_type, int bin_type, int locator, const void *in,
                      int64_t n, void *bins, int64_t num_bins,
                      int32_t *overflow);
+
+/* UniqueKernel (UniqueExtensions.cs:59-118): consecutive duplicates under
+ * Comparison<T> (CompareTo) removed in place, groups of `tile` elements run in
+ * sequence; returns the new length (-1 on bad arguments). */
+int64_t oracle_unique(int type, void *data, int64_t n, int64_t tile);
 
 /* Temp sizing on the CPU accelerator, in 32-bit ints
  * (RadixSortExtensions.cs:419-447, :384-404; ScanExtensions.cs:158-170). */

@@ -275,6 +275,95 @@ static void ScanErrors(Accelerator& accl) {
   CHECK(got[0] == 0 && got[99] == 198);
 }
 
+// ---- UniqueExtensionTests (UniqueExtensionTests.tt:36-90) -----------------------
+template <typename T> void UniqueTests(Accelerator& accl) {
+  namespace CO = ilgpu::ComparisonOperations;
+  for (int repeat : {1, 317, 1025}) {
+    for (int length : {1025, 70000}) {
+      std::vector<T> input((size_t)length), expected;
+      for (int i = 0; i < length; ++i) input[i] = (T)(i / repeat + 1);
+      for (const T& e : input)
+        if (expected.empty() || expected.back() != e) expected.push_back(e);
+      auto buf = accl.Allocate1D<T>(length);
+      buf->CopyFromCPU(input);
+      const int64_t result =
+          Unique<T, CO::Comparison<T>>(accl, accl.DefaultStream(), buf->View());
+      CHECK(result == (int64_t)expected.size());
+      CHECK(Verify(buf->GetAsArray1D(), expected));
+    }
+  }
+}
+static void UniqueErrors(Accelerator& accl) {
+  namespace CO = ilgpu::ComparisonOperations;
+  auto unique = CreateUnique<int32_t, CO::ComparisonInt32>(accl);
+  auto in = accl.Allocate1D<int32_t>(100);
+  auto out = accl.Allocate1D<int64_t>(1);
+  auto tmp = accl.Allocate1D<int32_t>(ComputeUniqueTempStorageSize<int32_t>(accl, 100));
+  auto& s = accl.DefaultStream();
+  EXPECT_THROW(unique(s, ArrayView<int32_t>(), out->View(), tmp->View()), ArgumentNullException);
+  EXPECT_THROW(unique(s, in->View(), ArrayView<int64_t>(), tmp->View()), ArgumentNullException);
+  EXPECT_THROW(unique(s, in->View(), out->View(), ArrayView<int32_t>()), ArgumentNullException);
+  EXPECT_THROW(unique(s, in->View(), out->View(), tmp->View().SubView(0, 1)),
+               ArgumentOutOfRangeException);
+}
+
+// ---- SequencerTests (SequencerTests.tt:56-200), InitializeTests, ReorderExtensionTests ----
+template <typename T, typename TSequencer> void SequencerTests(Accelerator& accl) {
+  for (int length : kArraySizes) {
+    auto buf = accl.Allocate1D<T>(length);
+    auto stream = accl.CreateStream();
+    ArrayView1D<T, Stride1D::Dense> view(buf->View());
+    Sequence(accl, *stream, view, TSequencer());
+    stream->Synchronize();
+    std::vector<T> expected((size_t)length);
+    for (int i = 0; i < length; ++i) expected[i] = (T)i;
+    CHECK(Verify(buf->GetAsArray1D(), expected));
+    RepeatedSequence(accl, *stream, view, 2, TSequencer());
+    stream->Synchronize();
+    for (int i = 0; i < length; ++i) expected[i] = (T)(i % 2);
+    CHECK(Verify(buf->GetAsArray1D(), expected));
+    BatchedSequence(accl, *stream, view, 2, TSequencer());
+    stream->Synchronize();
+    for (int i = 0; i < length; ++i) expected[i] = (T)(i / 2);
+    CHECK(Verify(buf->GetAsArray1D(), expected));
+    RepeatedBatchedSequence(accl, *stream, view, 2, 2, TSequencer());
+    stream->Synchronize();
+    for (int i = 0; i < length; ++i) expected[i] = (T)((i / 2) % 2);
+    CHECK(Verify(buf->GetAsArray1D(), expected));
+    EXPECT_THROW(RepeatedSequence(accl, *stream, view, 0, TSequencer()),
+                 ArgumentOutOfRangeException);
+    EXPECT_THROW(BatchedSequence(accl, *stream, view, 0, TSequencer()),
+                 ArgumentOutOfRangeException);
+  }
+}
+template <typename T> void InitializeAndReorderTests(Accelerator& accl) {
+  for (int length : kArraySizes) {
+    auto buf = accl.Allocate1D<T>(length);
+    auto target = accl.Allocate1D<T>(length);
+    auto order = accl.Allocate1D<Index1D>(length);
+    auto& s = accl.DefaultStream();
+    Initialize(accl, s, buf->View(), (T)42);
+    accl.Synchronize();
+    CHECK(Verify(buf->GetAsArray1D(), std::vector<T>((size_t)length, (T)42)));
+    // reverse through Reorder
+    const auto seq = ComputeSequence<T>(0, 1, length);
+    std::vector<Index1D> rev((size_t)length);
+    for (int i = 0; i < length; ++i) rev[i] = length - 1 - i;
+    buf->CopyFromCPU(seq);
+    order->CopyFromCPU(rev);
+    Reorder(accl, s, buf->View(), target->View(), order->View());
+    accl.Synchronize();
+    CHECK(Verify(target->GetAsArray1D(), ComputeInvertedSequence<T>(0, 1, length)));
+    if (length > 1) {
+      EXPECT_THROW(Reorder(accl, s, buf->View(), target->View(), order->View().SubView(0, length - 1)),
+                   ArgumentOutOfRangeException);
+      EXPECT_THROW(Reorder(accl, s, buf->View(), target->View().SubView(0, length - 1), order->View()),
+                   ArgumentOutOfRangeException);
+    }
+    EXPECT_THROW(Initialize(accl, s, ArrayView<T>(), (T)1), ArgumentNullException);
+  }
+}
+
 // ---- ReductionExtensionTests ----------------------------------------------------
 template <typename T, typename TOp> void ReduceTests(Accelerator& accl, int maxLength) {
   for (int length : kArraySizes) {
@@ -415,6 +504,19 @@ int main(int argc, char** argv) {
     RUN((HistogramTests<int64_t, int64_t>(accl)));
     RUN((HistogramTests<float, uint64_t>(accl)));
     RUN((HistogramTests<int16_t, int32_t>(accl)));
+    RUN(UniqueTests<int32_t>(accl));
+    RUN(UniqueTests<uint8_t>(accl));
+    RUN(UniqueTests<int64_t>(accl));
+    RUN(UniqueTests<float>(accl));
+    RUN(UniqueTests<double>(accl));
+    RUN(UniqueErrors(accl));
+    RUN((SequencerTests<int32_t, ilgpu::Sequencers::IndexSequencer>(accl)));
+    RUN((SequencerTests<int8_t, ilgpu::Sequencers::Int8Sequencer>(accl)));
+    RUN((SequencerTests<uint64_t, ilgpu::Sequencers::UInt64Sequencer>(accl)));
+    RUN((SequencerTests<double, ilgpu::Sequencers::DoubleSequencer>(accl)));
+    RUN(InitializeAndReorderTests<int32_t>(accl));
+    RUN(InitializeAndReorderTests<uint16_t>(accl));
+    RUN(InitializeAndReorderTests<double>(accl));
   }
   std::printf("%d test groups, %d failed checks\n", g_run, g_failed);
   return g_failed == 0 ? 0 : 1;

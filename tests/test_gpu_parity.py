@@ -594,3 +594,155 @@ def test_histogram_strided(num_bins, stride):
                              locator=O.LOCATOR_MODULO)
         assert np.array_equal(bins.numpy(), eb)
         assert ov.numpy()[0] == eo
+
+
+# -------------------------------------- unique, initialize, sequence, reorder
+def gpu_unique(values):
+    d = D.from_numpy(values)
+    out_len = D.zeros(1, np.int64)
+    capi.unique(d, out_len)
+    sync()
+    kept = int(out_len.numpy()[0])
+    return d.numpy()[:kept], d.numpy()[kept:], kept
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("repeat", [1, 317, 1025])
+def test_unique_reference_cases(dtype, repeat):
+    # UniqueExtensionTests.tt:48-67 (1025 elements) and :69-90 (more elements
+    # than one grid of groups covers; here: several tiles).
+    if np.dtype(dtype) == np.float16:
+        pytest.skip("values above 2048 are not exact in Half")
+    for length in (1025, 300001):
+        note("unique", np.dtype(dtype).name, repeat, length)
+        vals = np.repeat(np.arange(1, length // repeat + 2), repeat)[:length]
+        vals = (vals.astype(np.int64).astype(dtype) if np.dtype(dtype).kind in "iu"
+                else vals.astype(dtype))
+        kept, _, count = gpu_unique(vals)
+        expect = O.unique(vals)
+        assert count == expect.size
+        assert np.array_equal(kept, expect)
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.uint32, np.int64, np.float32, np.float64, np.float16])
+def test_unique_random_runs(dtype):
+    for n in [1, 2, 63, 64, 65, 8191, 8192, 8193, 1 << 20, (1 << 22) + 5]:
+        note("unique runs", np.dtype(dtype).name, n)
+        r = np.random.default_rng(n)
+        runs = r.integers(1, 6, size=n)
+        base = r.integers(0, 3, size=n)
+        vals = np.repeat(base, runs)[:n].astype(dtype)
+        if np.dtype(dtype).kind == "f" and n > 8:
+            vals[3:6] = np.nan               # a run of NaNs is one value
+            vals[6] = -0.0
+            vals[7] = 0.0                    # equal to -0.0
+        kept, _, count = gpu_unique(vals)
+        expect = O.unique(vals)
+        assert count == expect.size, n
+        assert np.array_equal(kept.view(np.uint8), expect.view(np.uint8)), n
+
+
+def test_unique_all_equal_and_all_distinct_large():
+    n = (1 << 24) + 3
+    kept, _, count = gpu_unique(np.full(n, 7, dtype=np.int32))
+    assert count == 1 and kept[0] == 7
+    seq = np.arange(n, dtype=np.uint32)
+    kept, _, count = gpu_unique(seq)
+    assert count == n and np.array_equal(kept, seq)
+
+
+def test_unique_unaligned_view():
+    vals = np.repeat(np.arange(5000, dtype=np.int32), 3)
+    base = D.from_numpy(np.concatenate([np.array([99], np.int32), vals]))
+    view = base.subview(1, vals.size)
+    out_len = D.zeros(1, np.int64)
+    capi.unique(view, out_len)
+    sync()
+    got = base.numpy()
+    assert got[0] == 99 and int(out_len.numpy()[0]) == 5000
+    assert np.array_equal(got[1:5001], np.arange(5000, dtype=np.int32))
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("n", ARRAY_SIZES + [100003])
+def test_sequence_reference_cases(dtype, n):
+    # SequencerTests.tt:56-96 and the repeated/batched forms.
+    d = D.zeros(n, dtype)
+    capi.sequence(d)
+    sync()
+    assert np.array_equal(d.numpy().view(np.uint8), O.sequence(n, dtype).view(np.uint8))
+    for seq_len, batch in [(5, 1), (n, 4), (7, 3)]:
+        capi.sequence(d, sequence_length=seq_len, batch_length=batch)
+        sync()
+        assert np.array_equal(d.numpy().view(np.uint8),
+                              O.sequence(n, dtype, seq_len, batch).view(np.uint8))
+
+
+def test_sequence_strided_and_errors():
+    phys = D.from_numpy(np.full(30, -1, dtype=np.int32))
+    capi.sequence(phys.strided(3))
+    sync()
+    got = phys.numpy()
+    assert np.array_equal(got[::3], np.arange(10, dtype=np.int32))
+    assert np.all(np.delete(got, np.arange(0, 30, 3)) == -1)
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.sequence(phys, sequence_length=0)
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.sequence(phys, batch_length=0)
+    with pytest.raises(capi.ArgumentNullError):
+        capi.sequence(D(0, np.int32))
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("n", [1, 5, 127, 4099, 1 << 20])
+def test_initialize(dtype, n):
+    value = np.array([3], dtype=np.int64).astype(dtype)[0] if np.dtype(dtype).kind != "f" else np.dtype(dtype).type(-1.5)
+    base = D.from_numpy(np.zeros(n + 2, dtype=dtype))
+    capi.initialize(base.subview(1, n), value)        # unaligned start: head/tail paths
+    sync()
+    got = base.numpy()
+    assert got[0] == 0 and got[-1] == 0
+    assert np.array_equal(got[1:-1], O.initialize(n, value))
+
+
+def test_initialize_strided_and_16_byte():
+    phys = D.from_numpy(np.zeros(40, dtype=np.uint16))
+    capi.initialize(phys.strided(4), 0xBEEF)
+    sync()
+    got = phys.numpy()
+    assert np.all(got[::4] == 0xBEEF) and np.all(np.delete(got, np.arange(0, 40, 4)) == 0)
+    pair = np.dtype([("a", np.uint64), ("b", np.uint64)])
+    d = D(1000, pair)
+    value = np.array([(1, 2)], dtype=pair)
+    capi.lib().ilgpu_hip_initialize(None, d.ptr, 1000, 1, 16, value.ctypes.data)
+    sync()
+    assert np.all(d.numpy() == value[0])
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.int64])
+def test_reorder(dtype):
+    for n in [1, 33, 1027, 1 << 18]:
+        src = np.random.default_rng(n).integers(0, 100, n).astype(dtype)
+        order = np.random.default_rng(n + 1).permutation(n).astype(np.int32)
+        tgt = D.zeros(n, dtype)
+        capi.reorder(D.from_numpy(src), tgt, D.from_numpy(order))
+        sync()
+        assert np.array_equal(tgt.numpy(), O.reorder(src, order))
+    # ReorderExtensions.cs:166-167: the order view must cover the source
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.reorder(D.zeros(10, dtype), D.zeros(10, dtype), D.zeros(5, np.int32))
+    # TransformExtensions.cs:324-331: the target must hold one element per index
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.reorder(D.zeros(10, dtype), D.zeros(9, dtype), D.zeros(10, np.int32))
+
+
+def test_sort_then_unique_pipeline():
+    # the pipeline the two primitives are used for: distinct keys of a column
+    keys = datagen.zipf_u32(1 << 22)
+    d = D.from_numpy(keys)
+    capi.radix_sort_keys(d)
+    out_len = D.zeros(1, np.int64)
+    capi.unique(d, out_len)
+    sync()
+    count = int(out_len.numpy()[0])
+    assert np.array_equal(d.numpy()[:count], np.unique(keys))

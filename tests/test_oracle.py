@@ -333,3 +333,75 @@ def test_temp_view_manager_alignment_rule(elem_bytes):
     assert got == (-2 if elem_bytes > 4 else 1 + rel)
     # Too small a temp view.
     assert O.temp_view_allocate(0, rel - 1 if rel > 1 else 0, elem_bytes, True, 1) == -1
+
+
+# ------------------------------------------- unique, sequence, reorder (oracle)
+def remove_consecutive_duplicates(a):
+    # UniqueExtensionTests.tt:36-46, the reference test's own expectation.
+    out = []
+    for x in a.tolist():
+        if not out or out[-1] != x:
+            out.append(x)
+    return np.array(out, dtype=a.dtype)
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("repeat", [1, 317, 1025])
+def test_unique_reference_cases(dtype, repeat):
+    # UniqueExtensionTests.tt:48-67: 1..length, each value repeated, cut at length.
+    if np.dtype(dtype) == np.float16:
+        pytest.skip("values above 2048 are not exact in Half")
+    length = 1025
+    vals = np.repeat(np.arange(1, length + 1), repeat)[:length]
+    if np.dtype(dtype).kind in "iu":
+        vals = vals.astype(np.int64).astype(dtype)     # wraps for 8-bit types, as (T)x
+    else:
+        vals = vals.astype(dtype)
+    expect = remove_consecutive_duplicates(vals)
+    for tile in (1, 16, 100, 4096):
+        assert np.array_equal(O.unique(vals, tile=tile), expect)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.uint16, np.int32, np.uint64])
+def test_unique_random_runs_any_tile(dtype):
+    for seed in range(5):
+        runs = rng(seed).integers(1, 9, size=300)
+        vals = np.repeat(rng(seed + 1).integers(0, 4, size=300), runs).astype(dtype)
+        keep = np.ones(vals.size, dtype=bool)
+        keep[1:] = vals[1:] != vals[:-1]            # first element of every run
+        for tile in (1, 7, 16, 1000):
+            assert np.array_equal(O.unique(vals, tile=tile), vals[keep])
+
+
+def test_unique_float_compare_to_semantics():
+    # CompareTo: every NaN equals every NaN, -0.0 equals +0.0; the FIRST of a run stays.
+    for dt in (np.float16, np.float32, np.float64):
+        nan2 = np.array([np.nan], dtype=dt)
+        nan2.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[nan2.itemsize])[0] |= 1
+        v = np.concatenate([np.array([np.nan], dt), nan2, np.array([-0.0, 0.0, 1.0, 1.0, np.inf, -np.inf, -np.inf], dt)])
+        out = O.unique(v, tile=3)
+        assert out.size == 5
+        assert np.isnan(out[0]) and np.signbit(out[1]) and out[1] == 0
+        assert out[2] == 1 and out[3] == np.inf and out[4] == -np.inf
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("n", ARRAY_SIZES)
+def test_sequence_reference_cases(dtype, n):
+    # SequencerTests.tt:56-96: expected[i] = (T)i.
+    expect = np.arange(n, dtype=np.int64)
+    expect = (expect.astype(np.uint64).astype(dtype) if np.dtype(dtype).kind == "u"
+              else expect.astype(dtype))
+    assert np.array_equal(O.sequence(n, dtype), expect)
+    # Repeated / Batched (SequenceExtensions.cs:163-171): closed form
+    got = O.sequence(n, dtype, sequence_length=5, batch_length=3)
+    for i in (0, n // 2, n - 1):
+        assert got[i] == np.dtype(dtype).type((i // 3) % 5)
+
+
+def test_reorder_is_a_gather():
+    src = rng(3).integers(0, 1000, 50).astype(np.int64)
+    order = rng(4).permutation(50).astype(np.int32)
+    out = O.reorder(src, order)
+    for i in range(50):
+        assert out[i] == src[order[i]]
