@@ -1,0 +1,169 @@
+"""GPU checks at the full baseline sizes, through properties that do not need a
+CPU pass over the data: sortedness plus a multiset checksum, encode-and-invert
+round trips, totals, and linearity.  Inputs are generated on the GPU by the
+seeded generators the benchmark uses."""
+import sys
+
+import numpy as np
+import pytest
+
+from ilgpu_amd import capi, datagen
+
+pytestmark = pytest.mark.gpu
+D = capi.DeviceArray
+
+
+def note(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def wrap(t, dtype):
+    import torch
+    return D(t.numel(), dtype, _bytes=t.view(torch.uint8))
+
+
+def u32(t):
+    import torch
+    return t.to(torch.int64) & 0xFFFFFFFF
+
+
+def test_sort_2p28_uniform_u32_sorted_and_same_multiset():
+    import torch
+    n = 1 << 28
+    note("sort 2^28 uniform u32")
+    src = datagen.uniform_u32_torch(n)
+    work = src.clone()
+    capi.radix_sort_keys(wrap(work, np.uint32))
+    torch.cuda.synchronize()
+    a, b = u32(work), u32(src)
+    assert bool((a[1:] >= a[:-1]).all().item())
+    # multiset equality through two independent checksums and the histogram of the top byte
+    assert int(a.sum().item()) == int(b.sum().item())
+    assert int((a * a % 1000003).sum().item()) == int((b * b % 1000003).sum().item())
+    assert torch.equal(torch.bincount(a >> 24, minlength=256), torch.bincount(b >> 24, minlength=256))
+    # idempotence: sorting the sorted array changes nothing
+    again = work.clone()
+    capi.radix_sort_keys(wrap(again, np.uint32))
+    torch.cuda.synchronize()
+    assert torch.equal(again, work)
+
+
+def test_sort_2p28_descending_is_reverse_of_ascending():
+    import torch
+    n = 1 << 28
+    note("sort 2^28 zipf u32 ascending vs descending")
+    src = datagen.zipf_u32_torch(n)
+    asc, desc = src.clone(), src.clone()
+    capi.radix_sort_keys(wrap(asc, np.uint32))
+    capi.radix_sort_keys(wrap(desc, np.uint32), descending=True)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.flip(desc, [0]), asc)
+
+
+def test_pairs_2p27_u64_index_values_invert_the_sort():
+    import torch
+    n = 1 << 27
+    note("pairs 2^27 u64 + index")
+    keys = datagen.splitmix64_torch(n)
+    work = keys.clone()
+    vals = torch.empty(n, dtype=torch.int32, device="cuda:0")
+    capi.radix_sort_pairs(wrap(work, np.uint64), wrap(vals, np.uint32), values_from_index=True)
+    torch.cuda.synchronize()
+    # values are a permutation that reproduces the output from the input
+    assert torch.equal(keys[vals.to(torch.int64)], work)
+    flipped = work ^ (-(1 << 63))
+    assert bool((flipped[1:] >= flipped[:-1]).all().item())
+    ties = work[1:] == work[:-1]
+    assert bool((vals[1:][ties] > vals[:-1][ties]).all().item())    # stable
+    assert int(torch.bincount(vals.to(torch.int64) >> 20).max().item()) == 1 << 20  # a permutation
+
+
+def test_scan_2p28_inclusive_exclusive_and_differences():
+    import torch
+    n = 1 << 28
+    note("scan 2^28 i32")
+    x = datagen.small_ints_i32_torch(n)
+    inc, exc = torch.empty_like(x), torch.empty_like(x)
+    capi.scan(wrap(x, np.int32), wrap(inc, np.int32), kind=capi.SCAN_INCLUSIVE)
+    capi.scan(wrap(x, np.int32), wrap(exc, np.int32), kind=capi.SCAN_EXCLUSIVE)
+    torch.cuda.synchronize()
+    assert torch.equal(inc - exc, x)                       # inclusive = exclusive + input
+    assert torch.equal(inc[1:] - inc[:-1], x[1:])          # differences give the input back
+    assert int(exc[0].item()) == 0
+    # values are 0..15, so the total stays below 2^31 and the int32 scan does not wrap
+    assert int(inc[-1].item()) == int(x.sum(dtype=torch.int64).item())
+
+
+def test_scan_2p28_max_is_monotone_and_bounded():
+    import torch
+    n = 1 << 28
+    x = datagen.gaussian_mixture_i32_torch(n)
+    out = torch.empty_like(x)
+    capi.scan(wrap(x, np.int32), wrap(out, np.int32), op=capi.OP_MAX, kind=capi.SCAN_INCLUSIVE)
+    torch.cuda.synchronize()
+    assert bool((out[1:] >= out[:-1]).all().item())
+    assert bool((out >= x).all().item())
+    assert int(out[-1].item()) == int(x.max().item())
+
+
+def test_reduce_2p28_f32_and_linearity():
+    import torch
+    n = 1 << 28
+    note("reduce 2^28 f32")
+    f = datagen.normal_f32_torch(n)
+    out = D.zeros(1, np.float32)
+    capi.reduce(wrap(f, np.float32), out)
+    torch.cuda.synchronize()
+    exact = float(f.sum(dtype=torch.float64).item())
+    got = float(out.numpy()[0])
+    # contract: within 1e-5 relative of the float64 sum (plus one float32 rounding)
+    assert abs(got - exact) <= 1e-5 * abs(exact) + abs(exact) * 2.0 ** -24
+    # the halves add up to the whole, in integers exactly
+    x = datagen.small_ints_i32_torch(n)
+    tot, lo, hi = D.zeros(1, np.int32), D.zeros(1, np.int32), D.zeros(1, np.int32)
+    d = wrap(x, np.int32)
+    capi.reduce(d, tot)
+    capi.reduce(d.subview(0, n // 2), lo)
+    capi.reduce(d.subview(n // 2, n // 2), hi)
+    torch.cuda.synchronize()
+    assert int(tot.numpy()[0]) == int(lo.numpy()[0]) + int(hi.numpy()[0])
+    assert int(tot.numpy()[0]) == int(x.sum(dtype=torch.int64).item())
+
+
+def test_histogram_2p30_u8_totals_and_accumulation():
+    import torch
+    n = 1 << 30
+    note("histogram 2^30 u8")
+    b = datagen.bytes_u8_torch(n)
+    bins, ov = D.zeros(256, np.int32), D.zeros(1, np.int32)
+    d = wrap(b, np.uint8)
+    capi.histogram(d, bins, ov)
+    torch.cuda.synchronize()
+    h1 = bins.numpy().astype(np.int64)
+    assert h1.sum() == n and ov.numpy()[0] == 0
+    expect = torch.zeros(256, dtype=torch.int64, device="cuda:0")
+    for c in range(4):
+        expect += torch.bincount(b[c << 28:(c + 1) << 28].to(torch.int64), minlength=256)
+    assert np.array_equal(h1, expect.cpu().numpy())
+    # a second call accumulates: twice the counts, and 2^31 total overflows no int32 bin
+    capi.histogram(d, bins, ov)
+    torch.cuda.synchronize()
+    assert np.array_equal(bins.numpy().astype(np.int64), 2 * h1) and ov.numpy()[0] == 0
+
+
+def test_unique_after_sort_2p28_counts_distinct_keys():
+    import torch
+    n = 1 << 28
+    note("sort + unique 2^28 zipf")
+    keys = datagen.zipf_u32_torch(n)
+    work = keys.clone()
+    d = wrap(work, np.uint32)
+    capi.radix_sort_keys(d)
+    count = D.zeros(1, np.int64)
+    capi.unique(d, count)
+    torch.cuda.synchronize()
+    kept = int(count.numpy()[0])
+    present = torch.bincount(u32(keys), minlength=1 << 16) > 0
+    assert kept == int(present.sum().item())
+    assert torch.equal(u32(work[:kept]), torch.nonzero(present).flatten())
