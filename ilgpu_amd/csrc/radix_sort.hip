@@ -61,6 +61,10 @@ constexpr int kSubLanes = 16;
 constexpr uint32_t kSubLaneMask = (1u << kSubLanes) - 1u;
 constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
 constexpr int kHistBlock = 512;
+#ifndef ILGPU_HIP_SORT_HIST_LDS_WORDS
+#define ILGPU_HIP_SORT_HIST_LDS_WORDS 16384
+#endif
+constexpr int kHistLdsWords = ILGPU_HIP_SORT_HIST_LDS_WORDS;
 constexpr uint32_t kStatusAggregate = 1u << 30;
 constexpr uint32_t kStatusPrefix = 2u << 30;
 constexpr uint32_t kStatusValueMask = (1u << 30) - 1u;
@@ -692,9 +696,9 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   if (rc != ILGPU_HIP_SUCCESS) return rc;
 
   {
-    int shift = 0;  // replicas: 32 KiB of LDS counters
+    int shift = 0;  // replicas: as many as kHistLdsWords of LDS counters hold
     while ((1 << (shift + 1)) <= 32 &&
-           ((passes * kRadix) << (shift + 1)) <= 8192)
+           ((passes * kRadix) << (shift + 1)) <= kHistLdsWords)
       ++shift;
     const size_t lds = (size_t)((passes * kRadix) << shift) * 4;
     int64_t blocks = div_up(div_up(a.n, Vec16<K>::N), kHistBlock);
