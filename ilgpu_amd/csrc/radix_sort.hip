@@ -65,10 +65,25 @@ constexpr int kHistBlock = 512;
 #define ILGPU_HIP_SORT_HIST_LDS_WORDS 16384
 #endif
 constexpr int kHistLdsWords = ILGPU_HIP_SORT_HIST_LDS_WORDS;
-constexpr uint32_t kStatusAggregate = 1u << 30;
-constexpr uint32_t kStatusPrefix = 2u << 30;
-constexpr uint32_t kStatusValueMask = (1u << 30) - 1u;
-constexpr int64_t kMaxSortLength = (1ll << 30) - 1;  // counts must fit 30 bits
+// Look-back status word of a (tile, digit): 0 = nothing published yet;
+// top bits 11 = the tile's own count in the low 30 bits (a count is at most a
+// tile); anything else = inclusive count over all tiles up to this one, plus
+// one.  An inclusive count is at most n <= 2^31 - 1, so count + 1 <= 2^31
+// never has both top bits set and is never 0.
+constexpr uint32_t kStatusAggregate = 3u << 30;
+constexpr uint32_t kStatusCountMask = (1u << 30) - 1u;
+__device__ __forceinline__ uint32_t status_aggregate(uint32_t count) {
+  return kStatusAggregate | count;
+}
+__device__ __forceinline__ uint32_t status_prefix(uint32_t inclusive) { return inclusive + 1u; }
+__device__ __forceinline__ bool status_is_aggregate(uint32_t w) {
+  return (w & kStatusAggregate) == kStatusAggregate;
+}
+// Value of a non-empty word and whether it ends the look-back.
+__device__ __forceinline__ uint32_t status_value(uint32_t w) {
+  return status_is_aggregate(w) ? w & kStatusCountMask : w - 1u;
+}
+constexpr int64_t kMaxSortLength = 0x7fffffffll;  // like the reference: int.MaxValue
 
 template <int KEY_BYTES> struct KeyOf;
 template <> struct KeyOf<1> { using type = uint8_t; };
@@ -396,7 +411,7 @@ __device__ __forceinline__ void sort_tile(
 #pragma unroll
     for (int s = 0; s < kSubTiles; ++s) count += s_slot[s * kRadix + tid] >> 16;
     __hip_atomic_store(&tile_status[tid],
-                       (tile == 0 ? kStatusPrefix : kStatusAggregate) | count,
+                       tile == 0 ? status_prefix(count) : status_aggregate(count),
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     inc = count;
 #pragma unroll
@@ -437,21 +452,21 @@ __device__ __forceinline__ void sort_tile(
       }
 #pragma unroll
       for (int u = 0; u < kLookback; ++u)
-        if (t - u < 0) s[u] = kStatusPrefix;
+        if (t - u < 0) s[u] = status_prefix(0u);
 #pragma unroll
       for (int u = 0; u < kLookback; ++u) {
         if (done) continue;
-        while ((s[u] & ~kStatusValueMask) == 0) {
+        while (s[u] == 0u) {
           __builtin_amdgcn_s_sleep(1);
           s[u] = __hip_atomic_load(&status[(int64_t)(t - u) * kRadix + tid],
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        before += s[u] & kStatusValueMask;
-        done = (s[u] & ~kStatusValueMask) == kStatusPrefix;
+        before += status_value(s[u]);
+        done = !status_is_aggregate(s[u]);
       }
     }
     if (tile > 0)
-      __hip_atomic_store(&tile_status[tid], kStatusPrefix | (before + count),
+      __hip_atomic_store(&tile_status[tid], status_prefix(before + count),
                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_global_off[tid] = excl[pass * kRadix + tid] + before - digit_start;
     if (tid == 0) *s_next_tile = (int)atomicAdd(ticket, 1u);

@@ -167,3 +167,24 @@ def test_unique_after_sort_2p28_counts_distinct_keys():
     present = torch.bincount(u32(keys), minlength=1 << 16) > 0
     assert kept == int(present.sum().item())
     assert torch.equal(u32(work[:kept]), torch.nonzero(present).flatten())
+
+
+def test_sort_beyond_2p30_keys():
+    # Per-digit inclusive counts pass 2^30 here (two key values only), which the
+    # look-back status words must carry; sortedness and the value counts pin
+    # the result.
+    import torch
+    n = (1 << 30) + 12345
+    note("sort 2^30 + 12345 u32, two distinct values")
+    idx = torch.arange(n, device="cuda:0", dtype=torch.int64)
+    src = torch.where(idx % (1 << 20) == 5,
+                      torch.tensor(7, device="cuda:0"), torch.tensor(0x01000003, device="cuda:0")).to(torch.int32)
+    del idx
+    sevens = int((src == 7).sum().item())
+    assert n - sevens > 1 << 30            # one digit's count passes 2^30
+    work = src.clone()
+    del src
+    capi.radix_sort_keys(wrap(work, np.uint32))
+    torch.cuda.synchronize()
+    assert bool((work[:sevens] == 7).all().item())
+    assert bool((work[sevens:] == 0x01000003).all().item())
