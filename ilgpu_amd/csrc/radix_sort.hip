@@ -98,14 +98,17 @@ template <> struct ValueOf<4> { using type = uint32_t; };
 template <> struct ValueOf<8> { using type = uint64_t; };
 template <> struct ValueOf<16> { using type = Bytes16; };
 
-// Keys per thread and tile.  Keys-only sorts take long tiles: the runs they
-// scatter are longer (fewer partial cache lines) and there are fewer tiles
-// to chain.  Values live in registers next to the keys, so pairs take the
-// short tile.  8-byte keys take two registers each: half the items, same
-// bytes per tile.
+// Keys per thread and tile.  Long tiles pay: the runs they scatter are longer
+// (fewer partial cache lines) and there are fewer tiles to chain.  Keys-only
+// sorts take 28 keys of up to 4 bytes or 14 of 8 bytes per thread.  Values
+// live in registers next to the keys: pairs with 4-byte keys stay at 16 items
+// (measured: longer is slower), pairs with 8-byte keys take 14 like the
+// keys-only tile unless the values are 16 bytes wide.
 constexpr int items_per_thread(int key_bytes, int value_bytes) {
-  const int items = value_bytes == 0 ? ILGPU_HIP_SORT_ITEMS : ILGPU_HIP_SORT_PAIR_ITEMS;
-  return key_bytes == 8 ? items / 2 : items;
+  if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_ITEMS;
+  if (key_bytes == 8)
+    return value_bytes <= 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_PAIR_ITEMS / 2;
+  return ILGPU_HIP_SORT_PAIR_ITEMS;
 }
 constexpr int tile_keys(int key_bytes, int value_bytes) {
   return kSortBlock * items_per_thread(key_bytes, value_bytes);
