@@ -14,7 +14,7 @@
 //             marks passes whose digit is the same for every key (they are
 //             skipped) and records which buffer each pass reads;
 //   pass x k  onesweep: a block takes a tile by ticket, ranks its keys
-//             (per-half-wave {peer mask, count} slots in LDS, so equal digits
+//             (per-quarter-wave {count, peer mask} slots in LDS, so equal digits
 //             keep memory order: every pass is stable), publishes
 //             its 256 digit counts, resolves the counts of all earlier tiles by
 //             decoupled look-back, stages the tile in digit order through LDS
@@ -40,7 +40,7 @@ namespace {
 constexpr int kRadix = 256;
 constexpr int kMaxPasses = 8;
 // Launch shape of the onesweep pass.  The block size fixes the number of
-// half-wave sub-tiles (and with it the LDS footprint of the ranking words);
+// quarter-wave sub-tiles (and with it the LDS footprint of the ranking slots);
 // items per thread fix the tile size.
 #ifndef ILGPU_HIP_SORT_BLOCK
 #define ILGPU_HIP_SORT_BLOCK 512
