@@ -176,14 +176,25 @@ template <typename T> struct Functor<T, ILGPU_HIP_OP_ADD> {
     }
   }
 };
+// Math.Max / Math.Min of the reference's MaxFloat/MinDouble... functors
+// (ScanReduceOperations.tt:36-72, IntrinsicMath.cs:111-112, 207-208): a NaN
+// operand wins (the first one if both are), and -0.0 < +0.0.  The hardware
+// maximum and minimum already order the signed zeros that way and return the
+// other operand for a NaN, so only the NaN selection is added.
+template <typename T> __device__ __forceinline__ T fp_hw_max(T a, T b) {
+  if constexpr (sizeof(T) == 4) return __builtin_fmaxf(a, b);
+  else return __builtin_fmax(a, b);
+}
+template <typename T> __device__ __forceinline__ T fp_hw_min(T a, T b) {
+  if constexpr (sizeof(T) == 4) return __builtin_fminf(a, b);
+  else return __builtin_fmin(a, b);
+}
 template <typename T> struct Functor<T, ILGPU_HIP_OP_MAX> {
   static __device__ __forceinline__ T identity() { return Limits<T>::lowest(); }
   static __device__ __forceinline__ T apply(T a, T b) {
     if constexpr (is_fp<T>::value) {
-      if (a != a) return a;
-      if (b != b) return b;
-      if (a == b) return fp_signbit(a) ? b : a;
-      return a > b ? a : b;
+      const T m = fp_hw_max(a, b);
+      return a != a ? a : (b != b ? b : m);
     } else {
       return a > b ? a : b;
     }
@@ -193,10 +204,8 @@ template <typename T> struct Functor<T, ILGPU_HIP_OP_MIN> {
   static __device__ __forceinline__ T identity() { return Limits<T>::highest(); }
   static __device__ __forceinline__ T apply(T a, T b) {
     if constexpr (is_fp<T>::value) {
-      if (a != a) return a;
-      if (b != b) return b;
-      if (a == b) return fp_signbit(a) ? a : b;
-      return a < b ? a : b;
+      const T m = fp_hw_min(a, b);
+      return a != a ? a : (b != b ? b : m);
     } else {
       return a < b ? a : b;
     }

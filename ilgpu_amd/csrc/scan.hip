@@ -20,7 +20,7 @@
 // started.  Status words are read and written with agent-scope atomics: the
 // eight XCDs of the device have separate L2s.
 //   4-byte T: one 64-bit word {flag, value} per tile;
-//   8-byte T: a flag word (release/acquire) and two value slots per tile.
+//   8-byte T: two such words per tile, one per half of the value.
 //
 // Algorithmic HBM traffic: 2 * n * sizeof(T) bytes (status words: 8 B/tile).
 #include "kernels.hpp"
@@ -90,29 +90,32 @@ template <typename T> struct TileState<T, 4> {
   }
 };
 
+// 8-byte values: two 64-bit words per tile, {flag, low half} and {flag, high
+// half}, each written and read with one relaxed atomic.  A tile writes each
+// state (aggregate, then prefix) once, so two words with the same flag hold
+// the halves of the same value; a reader that catches the words in different
+// states reads again.  No fences: an agent-scope release would write back the
+// whole L2 of the XCD for every tile.
 template <typename T> struct TileState<T, 8> {
-  uint32_t* flags;
-  uint64_t* aggregates;
-  uint64_t* prefixes;
+  uint64_t* low;
+  uint64_t* high;
   __device__ __forceinline__ void publish(int tile, uint32_t flag, T v) const {
-    uint64_t* slot = flag == kFlagPrefix ? prefixes : aggregates;
-    __hip_atomic_store(&slot[tile], to_bits(v), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&flags[tile], flag, __ATOMIC_RELEASE,
-                       __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t bits = to_bits(v);
+    __hip_atomic_store(&low[tile], ((uint64_t)flag << 32) | (uint32_t)bits,
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&high[tile], ((uint64_t)flag << 32) | (bits >> 32),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __device__ __forceinline__ uint32_t wait(int tile, T* v) const {
-    uint32_t f;
+    uint64_t lo, hi;
     while (true) {
-      f = __hip_atomic_load(&flags[tile], __ATOMIC_ACQUIRE,
-                            __HIP_MEMORY_SCOPE_AGENT);
-      if (f != kFlagInvalid) break;
+      lo = __hip_atomic_load(&low[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      hi = __hip_atomic_load(&high[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((uint32_t)(lo >> 32) != kFlagInvalid && (lo >> 32) == (hi >> 32)) break;
       __builtin_amdgcn_s_sleep(1);
     }
-    const uint64_t* slot = f == kFlagPrefix ? prefixes : aggregates;
-    *v = from_bits<T>(__hip_atomic_load(&slot[tile], __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT));
-    return f;
+    *v = from_bits<T>((uint64_t)(uint32_t)lo | (hi << 32));
+    return (uint32_t)(lo >> 32);
   }
 };
 
@@ -435,11 +438,9 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t in_stride,
     st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
     zero_words = (kHeaderBytes + tiles * 8) / 4;
   } else {
-    const int64_t flag_bytes = align_up(tiles * 4, 256);
-    st.flags = reinterpret_cast<uint32_t*>(base + kHeaderBytes);
-    st.aggregates = reinterpret_cast<uint64_t*>(base + kHeaderBytes + flag_bytes);
-    st.prefixes = st.aggregates + tiles;
-    zero_words = (kHeaderBytes + flag_bytes) / 4;
+    st.low = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
+    st.high = st.low + tiles;
+    zero_words = (kHeaderBytes + tiles * 16) / 4;
   }
   int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
                                  zero_words);
@@ -504,7 +505,7 @@ int64_t scan_temp_bytes(int64_t n, int elem_bytes) {
     return 256 + kHeaderBytes + tiles * 8;
   }
   const int64_t tiles = num_tiles<uint64_t>(n);
-  return 256 + kHeaderBytes + align_up(tiles * 4, 256) + tiles * 16;
+  return 256 + kHeaderBytes + tiles * 16;
 }
 
 int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,

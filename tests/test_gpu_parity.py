@@ -746,3 +746,26 @@ def test_sort_then_unique_pipeline():
     sync()
     count = int(out_len.numpy()[0])
     assert np.array_equal(d.numpy()[:count], np.unique(keys))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("op", [capi.OP_MAX, capi.OP_MIN])
+def test_scan_float_max_min_signed_zero_and_nan(dtype, op):
+    # Math.Max/Math.Min (IntrinsicMath.cs:111-112, 207-208): -0.0 < +0.0, and
+    # from the first NaN on every result is NaN.
+    for n in [64, 5000, 300000]:
+        r = np.random.default_rng(n)
+        v = r.integers(-3, 3, n).astype(dtype)
+        v[v == 0] = np.where(r.integers(0, 2, int((v == 0).sum())) == 0, 0.0, -0.0)
+        d_in, d_out = D.from_numpy(v), D.zeros(n, dtype)
+        capi.scan(d_in, d_out, op=op, kind=capi.SCAN_INCLUSIVE)
+        sync()
+        expect = O.scan(v, op=op, inclusive=True)
+        assert np.array_equal(d_out.numpy().view(np.uint8), expect.view(np.uint8)), n
+        w = v.copy()
+        w[n // 2] = np.nan
+        capi.scan(D.from_numpy(w), d_out, op=op, kind=capi.SCAN_INCLUSIVE)
+        sync()
+        got = d_out.numpy()
+        assert np.array_equal(got[: n // 2].view(np.uint8), expect[: n // 2].view(np.uint8))
+        assert np.isnan(got[n // 2:]).all()
