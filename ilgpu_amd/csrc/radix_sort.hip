@@ -103,12 +103,11 @@ template <> struct ValueOf<16> { using type = Bytes16; };
 // sorts take 28 keys of up to 4 bytes or 14 of 8 bytes per thread.  Values
 // live in registers next to the keys: pairs with 4-byte keys stay at 16 items
 // (measured: longer is slower), pairs with 8-byte keys take 14 like the
-// keys-only tile unless the values are 16 bytes wide.
+// keys-only tile, and 16-byte values (four registers each) take 8.
 constexpr int items_per_thread(int key_bytes, int value_bytes) {
   if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_ITEMS;
-  if (key_bytes == 8)
-    return value_bytes <= 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_PAIR_ITEMS / 2;
-  return ILGPU_HIP_SORT_PAIR_ITEMS;
+  if (value_bytes == 16) return ILGPU_HIP_SORT_PAIR_ITEMS / 2;
+  return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_PAIR_ITEMS;
 }
 constexpr int tile_keys(int key_bytes, int value_bytes) {
   return kSortBlock * items_per_thread(key_bytes, value_bytes);
