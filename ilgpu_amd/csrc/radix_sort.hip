@@ -31,6 +31,8 @@
 //
 // Algorithmic HBM traffic for n keys of k bytes, values of v bytes and P
 // executed passes: n * (k * (2P + 1) + v * 2P) bytes.
+#include <atomic>
+
 #include "kernels.hpp"
 
 namespace ilgpu_hip {
@@ -739,10 +741,16 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
     if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true>;
   }
-  int per_cu = 0;
-  ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
-      &per_cu, pass_kernel, kSortBlock, 0));
-  if (per_cu < 1) per_cu = 1;
+  // Resident blocks per CU of this instantiation: asked once per process and
+  // kernel (the query costs microseconds, which small sorts would feel).
+  static std::atomic<int> cached_per_cu[2] = {{0}, {0}};
+  int per_cu = cached_per_cu[float_keys ? 1 : 0].load(std::memory_order_relaxed);
+  if (per_cu == 0) {
+    ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+        &per_cu, pass_kernel, kSortBlock, 0));
+    if (per_cu < 1) per_cu = 1;
+    cached_per_cu[float_keys ? 1 : 0].store(per_cu, std::memory_order_relaxed);
+  }
   int64_t grid = (int64_t)cus * per_cu;
   if (grid > L.tiles) grid = L.tiles;
   for (int p = 0; p < passes; ++p) {
