@@ -769,3 +769,51 @@ def test_scan_float_max_min_signed_zero_and_nan(dtype, op):
         got = d_out.numpy()
         assert np.array_equal(got[: n // 2].view(np.uint8), expect[: n // 2].view(np.uint8))
         assert np.isnan(got[n // 2:]).all()
+
+
+# ------------------------------------------------------------- tile boundaries
+# Lengths just below, at and just above one and two tiles of every tile shape
+# the pass kernel uses (512 threads x 28, 16, 14 or 8 items).
+TILE_EDGE_SIZES = sorted({t * m + d for t in (4096, 7168, 8192, 14336) for m in (1, 2)
+                          for d in (-1, 0, 1)})
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.uint32, np.uint64, np.float64])
+def test_sort_keys_tile_edges(dtype):
+    for n in TILE_EDGE_SIZES:
+        note("sort edge", np.dtype(dtype).name, n)
+        keys = (random_float_bits(dtype, n, seed=n) if np.dtype(dtype).kind == "f"
+                else random_ints(dtype, n, seed=n))
+        d = D.from_numpy(keys)
+        capi.radix_sort_keys(d)
+        sync()
+        assert np.array_equal(d.numpy().view(np.uint8), O.radix_sort(keys).view(np.uint8)), n
+
+
+@pytest.mark.parametrize("kdt,vdt", [(np.uint32, np.uint32), (np.uint64, np.uint32),
+                                     (np.uint32, np.uint64), (np.uint16, np.uint8)])
+def test_sort_pairs_tile_edges(kdt, vdt):
+    for n in TILE_EDGE_SIZES:
+        note("pairs edge", np.dtype(kdt).name, np.dtype(vdt).name, n)
+        keys = random_ints(kdt, n, seed=n, lo=0, hi=500)        # duplicates: stability matters
+        vals = (np.arange(n, dtype=np.uint64) * 7 + 3).astype(vdt)
+        dk, dv = D.from_numpy(keys), D.from_numpy(vals)
+        capi.radix_sort_pairs(dk, dv)
+        sync()
+        ek, ev = O.radix_sort_pairs(keys, vals)
+        assert np.array_equal(dk.numpy(), ek) and np.array_equal(dv.numpy(), ev), n
+
+
+def test_sort_pairs_16_byte_values_tile_edges():
+    pair = np.dtype([("a", np.uint64), ("b", np.uint64)])
+    for n in TILE_EDGE_SIZES:
+        keys = random_ints(np.uint32, n, seed=n, lo=0, hi=300)
+        vals = np.zeros(n, dtype=pair)
+        vals["a"] = np.arange(n)
+        vals["b"] = ~np.arange(n, dtype=np.uint64)
+        dk, dv = D.from_numpy(keys), D.from_numpy(vals)
+        capi.radix_sort_pairs(dk, dv)
+        sync()
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(dk.numpy(), keys[order]), n
+        assert np.array_equal(dv.numpy(), vals[order]), n
