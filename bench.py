@@ -90,6 +90,18 @@ MEASURED_TRAFFIC_BYTES = {
     # (kernel, log2 n): bytes per launch
     ("onesweep_kernel<4,0>", 28): 2.475e9,
 }
+# The same for the other workloads at their default sizes, keyed by bench name.
+MEASURED_EXTRA_TRAFFIC_BYTES = {
+    "scan_exclusive_add_i32_2^28": 2.154e9,
+    "reduce_add_f32_2^28": 1.074e9,
+    "histogram_u8_256bins_2^30": 1.075e9,
+    "histogram_i32_4096bins_2^28": 1.091e9,
+    "radix_sort_pairs_u64_u32_2^27": 3.761e9,
+    "unique_i32_all_distinct_2^28": 2.159e9,
+    "sequence_i32_2^28": 1.074e9,
+    "initialize_i32_2^28": 1.074e9,
+    "reorder_u32_random_permutation_2^28": 3.639e10,
+}
 
 
 def roofline(achieved_gbs, traffic=None):
@@ -250,8 +262,9 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
         entry = {"ms_per_step": round(t, 4),
                  "algorithmic_gbs": round(algo_bytes / (t * 1e-3) / 1e9, 1),
                  "frac_of_hbm_peak": round(algo_bytes / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                 "roofline": dict(roofline(k_gbs), kernel=kernel,
-                                  avg_launch_ms=round(k_ms, 4))}
+                 "roofline": dict(roofline(k_gbs, MEASURED_EXTRA_TRAFFIC_BYTES.get(name)
+                                           if args.log2n == 28 else None),
+                                  kernel=kernel, avg_launch_ms=round(k_ms, 4))}
         out[name] = entry
         log(f"[bench] {name}: {t:.3f} ms/step, {entry['algorithmic_gbs']:.0f} GB/s "
             f"({100 * entry['frac_of_hbm_peak']:.1f}% of peak)")
