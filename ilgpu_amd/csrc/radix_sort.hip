@@ -426,8 +426,13 @@ __device__ __forceinline__ void sort_tile(
     if (lane == kWaveSize - 1) s_scan[wave] = inc;
   }
   __syncthreads();
+  // Digit threads: run starts, and the first step of the look-back is put in
+  // flight; it is consumed after the keys are staged, so its round trip
+  // overlaps the position and staging work of the whole block.
+  uint32_t digit_start = 0;
+  uint32_t first_step[kLookback];
   if (tid < kRadix) {
-    uint32_t digit_start = inc - count;
+    digit_start = inc - count;
     for (int w = 0; w < wave; ++w) digit_start += s_scan[w];
     // Tile-local position of the first key of every (sub-tile, digit) run.
     {
@@ -439,21 +444,50 @@ __device__ __forceinline__ void sort_tile(
         run += t;
       }
     }
+#pragma unroll
+    for (int u = 0; u < kLookback; ++u) {
+      const int idx = tile - 1 - u < 0 ? 0 : tile - 1 - u;
+      first_step[u] = __hip_atomic_load(&status[(int64_t)idx * kRadix + tid],
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  __syncthreads();
 
+  // Tile-local position of every key; afterwards the slots are dead and the
+  // same LDS bytes stage the keys in digit order.
+#pragma unroll
+  for (int j = 0; j < kItems; j += 2) {
+    const uint32_t p0 = my_slots[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
+    const uint32_t p1 = my_slots[item_digit(j + 1)] + (packed[j / 2] >> 16);
+    packed[j / 2] = p0 | (p1 << 16);
+    if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kItems; ++j)
+    s_keys[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = key[j];
+
+  if (tid < kRadix) {
     // Keys with this digit in earlier tiles: walk back over the status words,
     // kLookback tiles per step.  The loads of a step are unconditional (index
     // clamped) so that they are in flight together; positions in front of
     // tile 0 read as an empty inclusive prefix.
     uint32_t before = 0;
     bool done = tile == 0;
+    bool preloaded = true;
     for (int t = tile - 1; !done; t -= kLookback) {
       uint32_t s[kLookback];
 #pragma unroll
       for (int u = 0; u < kLookback; ++u) {
-        const int idx = t - u < 0 ? 0 : t - u;
-        s[u] = __hip_atomic_load(&status[(int64_t)idx * kRadix + tid],
-                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (preloaded) {
+          s[u] = first_step[u];
+        } else {
+          const int idx = t - u < 0 ? 0 : t - u;
+          s[u] = __hip_atomic_load(&status[(int64_t)idx * kRadix + tid],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
+      preloaded = false;
 #pragma unroll
       for (int u = 0; u < kLookback; ++u)
         if (t - u < 0) s[u] = status_prefix(0u);
@@ -477,21 +511,6 @@ __device__ __forceinline__ void sort_tile(
   }
   __syncthreads();
   next_tile = *s_next_tile;
-
-  // Tile-local position of every key; afterwards the slots are dead and the
-  // same LDS bytes stage the keys in digit order.
-#pragma unroll
-  for (int j = 0; j < kItems; j += 2) {
-    const uint32_t p0 = my_slots[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
-    const uint32_t p1 = my_slots[item_digit(j + 1)] + (packed[j / 2] >> 16);
-    packed[j / 2] = p0 | (p1 << 16);
-    if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
-  }
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < kItems; ++j)
-    s_keys[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = key[j];
-  __syncthreads();
 
   // The key registers are free: fetch the next tile during the write-out.
   {
