@@ -309,9 +309,7 @@ __device__ __forceinline__ void load_tile_keys(
 #define ILGPU_HIP_SORT_WAVES_PER_EU 4
 #endif
 
-// Sorts one tile by the digit of `pass` and scatters it.  On return `key`
-// holds the keys of the block's next tile (ticket in `next_tile`), loaded
-// while this tile was written out.
+// Sorts one tile by the digit of `pass` and scatters it.
 template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL>
 __device__ __forceinline__ void sort_tile(
     typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
@@ -320,9 +318,7 @@ __device__ __forceinline__ void sort_tile(
     typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
     int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
     const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
-    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan,
-    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int64_t n,
-    uint32_t* ticket, int num_tiles, int* s_next_tile, int& next_tile) {
+    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
@@ -507,23 +503,8 @@ __device__ __forceinline__ void sort_tile(
       __hip_atomic_store(&tile_status[tid], status_prefix(before + count),
                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_global_off[tid] = excl[pass * kRadix + tid] + before - digit_start;
-    if (tid == 0) *s_next_tile = (int)atomicAdd(ticket, 1u);
   }
   __syncthreads();
-  next_tile = *s_next_tile;
-
-  // The key registers are free: fetch the next tile during the write-out.
-  {
-    const int64_t next_base = (int64_t)next_tile * TileCfg::kTile;
-    const int64_t remaining = n - next_base;
-    if (next_tile < num_tiles && remaining >= TileCfg::kTile)
-      load_tile_keys<KEY_BYTES, kItems, true>(src_keys, next_base, TileCfg::kTile, first_local, key);
-    else
-      load_tile_keys<KEY_BYTES, kItems, false>(
-          src_keys, next_base,
-          next_tile < num_tiles && remaining > 0 ? (int)remaining : 0,
-          first_local, key);
-  }
 
   uint32_t gpos[kPairs ? kItems : 1];
   asm volatile("" : "+v"(tid));
@@ -579,7 +560,7 @@ void onesweep_kernel(
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[TileCfg::kStageBytes];
   __shared__ uint32_t s_global_off[kRadix];
   __shared__ uint32_t s_scan[kRadix / kWaveSize];
-  __shared__ int s_tile[2];
+  __shared__ int s_tile;
 
   if (plan->skip[pass]) return;
   const bool src_alt = plan->src_is_alt[pass] != 0;
@@ -597,38 +578,36 @@ void onesweep_kernel(
     return remaining >= kTile ? kTile : (remaining > 0 ? (int)remaining : 0);
   };
 
-  if (tid == 0) s_tile[0] = (int)atomicAdd(ticket, 1u);
-  __syncthreads();
-  int tile = s_tile[0];
-  K key[kItems];
-  if (tile < num_tiles) {
+  // A block draws its next tile only when it is about to start it: the time
+  // between a tile's ticket and the publication of its digit counts is what
+  // every later tile's look-back waits for.  (Drawing it earlier, to load the
+  // next keys during the write-out, measured 3 to 12 % slower.)  The key loads
+  // fly while the ranking slots are cleared.
+  while (true) {
+    if (tid == 0) s_tile = (int)atomicAdd(ticket, 1u);
+    __syncthreads();  // also: the previous tile's staged keys have been read
+    const int tile = s_tile;
+    if (tile >= num_tiles) break;
+    const int64_t tile_base = (int64_t)tile * kTile;
     const int valid = valid_keys(tile);
-    if (valid == kTile) load_tile_keys<KEY_BYTES, kItems, true>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
-    else load_tile_keys<KEY_BYTES, kItems, false>(src_keys, (int64_t)tile * kTile, valid, first_local, key);
-  }
-  while (tile < num_tiles) {
-    {  // clear the mask and count words
+    K key[kItems];
+    if (valid == kTile) load_tile_keys<KEY_BYTES, kItems, true>(src_keys, tile_base, valid, first_local, key);
+    else load_tile_keys<KEY_BYTES, kItems, false>(src_keys, tile_base, valid, first_local, key);
+    {  // clear the ranking slots
       uint4* z = reinterpret_cast<uint4*>(s_stage);
       for (int i = tid; i < TileCfg::kSlotBytes / 16; i += kSortBlock)
         z[i] = make_uint4(0u, 0u, 0u, 0u);
     }
     __syncthreads();
-    const int64_t tile_base = (int64_t)tile * kTile;
-    const int valid = valid_keys(tile);
-    int next = num_tiles;
     if (valid == kTile) {
       sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, true>(
           key, dst_keys, src_vals, dst_vals, tile_base, kTile, tile, pass, xf,
-          excl, status, make_index, s_stage, s_global_off, s_scan,
-          src_keys, n, ticket, num_tiles, &s_tile[1], next);
+          excl, status, make_index, s_stage, s_global_off, s_scan);
     } else {
       sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false>(
           key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
-          excl, status, make_index, s_stage, s_global_off, s_scan,
-          src_keys, n, ticket, num_tiles, &s_tile[1], next);
+          excl, status, make_index, s_stage, s_global_off, s_scan);
     }
-    tile = next;
-    __syncthreads();  // LDS is reused by the next tile
   }
 }
 
