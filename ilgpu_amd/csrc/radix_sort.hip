@@ -48,10 +48,10 @@ constexpr int kMaxPasses = 8;
 #define ILGPU_HIP_SORT_BLOCK 512
 #endif
 #ifndef ILGPU_HIP_SORT_ITEMS
-#define ILGPU_HIP_SORT_ITEMS 28
+#define ILGPU_HIP_SORT_ITEMS 36
 #endif
-#ifndef ILGPU_HIP_SORT_PAIR_ITEMS
-#define ILGPU_HIP_SORT_PAIR_ITEMS 16
+#ifndef ILGPU_HIP_SORT_ITEMS8
+#define ILGPU_HIP_SORT_ITEMS8 18
 #endif
 #ifndef ILGPU_HIP_SORT_LOOKBACK
 #define ILGPU_HIP_SORT_LOOKBACK 4
@@ -102,14 +102,16 @@ template <> struct ValueOf<16> { using type = Bytes16; };
 
 // Keys per thread and tile.  Long tiles pay: the runs they scatter are longer
 // (fewer partial cache lines) and there are fewer tiles to chain.  Keys-only
-// sorts take 28 keys of up to 4 bytes or 14 of 8 bytes per thread.  Values
-// live in registers next to the keys: pairs with 4-byte keys stay at 16 items
-// (measured: longer is slower), pairs with 8-byte keys take 14 like the
-// keys-only tile, and 16-byte values (four registers each) take 8.
+// sorts take 36 keys of up to 4 bytes or 18 of 8 bytes per thread: the most
+// that lets two blocks share a compute unit's 160 KiB of LDS.  Values live in
+// registers next to the keys, which caps pairs lower, by the registers one
+// pair takes: 20 items at two (key and value of up to 4 bytes each), 16 at
+// three, 14 at four, 8 with 16-byte values.  (Measured at 12 to 24 items.)
 constexpr int items_per_thread(int key_bytes, int value_bytes) {
-  if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_ITEMS;
-  if (value_bytes == 16) return ILGPU_HIP_SORT_PAIR_ITEMS / 2;
-  return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS / 2 : ILGPU_HIP_SORT_PAIR_ITEMS;
+  if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS8 : ILGPU_HIP_SORT_ITEMS;
+  if (value_bytes == 16) return 8;
+  const int registers = (key_bytes == 8 ? 2 : 1) + (value_bytes == 8 ? 2 : 1);
+  return registers == 2 ? 20 : registers == 3 ? 16 : 14;
 }
 constexpr int tile_keys(int key_bytes, int value_bytes) {
   return kSortBlock * items_per_thread(key_bytes, value_bytes);

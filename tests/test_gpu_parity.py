@@ -773,8 +773,9 @@ def test_scan_float_max_min_signed_zero_and_nan(dtype, op):
 
 # ------------------------------------------------------------- tile boundaries
 # Lengths just below, at and just above one and two tiles of every tile shape
-# the pass kernel uses (512 threads x 28, 16, 14 or 8 items).
-TILE_EDGE_SIZES = sorted({t * m + d for t in (4096, 7168, 8192, 14336) for m in (1, 2)
+# the pass kernel uses (512 threads x 36, 20, 18, 16, 14 or 8 items).
+TILE_EDGE_SIZES = sorted({t * m + d for t in (4096, 7168, 8192, 9216, 10240, 18432)
+                          for m in (1, 2)
                           for d in (-1, 0, 1)})
 
 
