@@ -419,7 +419,16 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
               lambda: capi.reorder(wrap(source, np.uint32), d, wrap(perm, np.int32)),
               12.0 * n28, "reorder")
     e["verified"] = bool((work == source[perm.to(torch.int64)]).all().item())
-    del work, perm, source
+    # Transform: i32 -> -i32 (n * 8 bytes) and the widening i32 -> i64 (n * 12 bytes).
+    d_src = wrap(source, np.int32)
+    e = timed("transform_negate_i32_2^28", nothing,
+              lambda: capi.transform(d_src, d, capi.TRANSFORM_NEGATE), 8.0 * n28, "transform")
+    e["verified"] = bool((work == -source).all().item())
+    wide = torch.empty(n28, dtype=torch.int64, device="cuda:0")
+    e = timed("transform_i32_to_i64_2^28", nothing,
+              lambda: capi.transform(d_src, wrap(wide, np.int64)), 12.0 * n28, "transform")
+    e["verified"] = bool((wide == source.to(torch.int64)).all().item())
+    del work, perm, source, wide
     return out
 
 

@@ -35,6 +35,8 @@ SCAN_INCLUSIVE, SCAN_EXCLUSIVE = 0, 1
 SORT_DESCENDING, SORT_FLOAT_TOTAL_ORDER = 1, 2
 VALUES_FROM_VIEW, VALUES_FROM_INDEX = 0, 1
 LOCATOR_IDENTITY, LOCATOR_MODULO = 0, 1
+(TRANSFORM_CONVERT, TRANSFORM_NEGATE, TRANSFORM_BIT_COMPLEMENT,
+ TRANSFORM_MULTIPLY) = 0, 1, 2, 3
 
 EXPORTS = [
     "ilgpu_hip_version", "ilgpu_hip_status_string",
@@ -46,6 +48,7 @@ EXPORTS = [
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
     "ilgpu_hip_unique_temp_bytes", "ilgpu_hip_unique", "ilgpu_hip_initialize",
     "ilgpu_hip_sequence", "ilgpu_hip_reorder",
+    "ilgpu_hip_transform", "ilgpu_hip_reorder_transform",
 ]
 
 _NP_TO_TYPE = {
@@ -134,6 +137,8 @@ def lib() -> ctypes.CDLL:
         L.ilgpu_hip_initialize.argtypes = [vp, vp, i64, i64, i32, vp]
         L.ilgpu_hip_sequence.argtypes = [vp, vp, i64, i64, i32, i64, i64]
         L.ilgpu_hip_reorder.argtypes = [vp, vp, i64, vp, i64, vp, i64, i32]
+        L.ilgpu_hip_transform.argtypes = [vp, vp, i64, i64, i32, vp, i64, i64, i32, i32, i64]
+        L.ilgpu_hip_reorder_transform.argtypes = [vp, vp, i64, i32, vp, i64, i32, vp, i64, i32, i64]
         L.ilgpu_hip_reduce.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64, vp, i64]
         L.ilgpu_hip_histogram.argtypes = [vp, vp, i64, i64, i32, vp, i64, i32,
                                           i32, vp]
@@ -370,3 +375,23 @@ def reorder(source: DeviceArray, target: DeviceArray, order: DeviceArray, *,
     check(lib().ilgpu_hip_reorder(
         _stream_ptr(stream), source.ptr, source.length, target.ptr,
         target.length, order.ptr, order.length, source.dtype.itemsize))
+
+
+def transform(source: DeviceArray, target: DeviceArray,
+              transformer: int = TRANSFORM_CONVERT, factor: int = 0, *,
+              stream=None) -> None:
+    """Transform: target[i] = (TTarget)op(source[i])."""
+    check(lib().ilgpu_hip_transform(
+        _stream_ptr(stream), source.ptr, source.length, source.stride,
+        source.type_code, target.ptr, target.length, target.stride,
+        target.type_code, transformer, factor))
+
+
+def reorder_transform(source: DeviceArray, target: DeviceArray,
+                      order: DeviceArray, transformer: int = TRANSFORM_CONVERT,
+                      factor: int = 0, *, stream=None) -> None:
+    """ReorderTransform: target[i] = (TTarget)op(source[order[i]])."""
+    check(lib().ilgpu_hip_reorder_transform(
+        _stream_ptr(stream), source.ptr, source.length, source.type_code,
+        target.ptr, target.length, target.type_code, order.ptr, order.length,
+        transformer, factor))

@@ -438,4 +438,66 @@ int32_t ilgpu_hip_reorder(ilgpu_hip_stream_t stream, const void* source,
                         order_length, elem_bytes);
 }
 
+/* ---- transform, reorder-transform --------------------------------------- */
+
+static int32_t check_transformer(int32_t source_type, int32_t target_type,
+                                 int32_t transformer) {
+  if (elem_size(source_type) < 0 || elem_size(target_type) < 0)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (transformer < ILGPU_HIP_TRANSFORM_CONVERT ||
+      transformer > ILGPU_HIP_TRANSFORM_MULTIPLY)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const bool float_source = source_type >= ILGPU_HIP_F16;
+  const bool float_target = target_type >= ILGPU_HIP_F16;
+  if (float_source && !float_target) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (float_source && transformer == ILGPU_HIP_TRANSFORM_BIT_COMPLEMENT)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  return ILGPU_HIP_SUCCESS;
+}
+
+int32_t ilgpu_hip_transform(ilgpu_hip_stream_t stream, const void* source,
+                            int64_t source_length, int64_t source_stride,
+                            int32_t source_type, void* target,
+                            int64_t target_length, int64_t target_stride,
+                            int32_t target_type, int32_t transformer,
+                            int64_t factor) {
+  /* TransformExtensions.cs:304-317. */
+  const int32_t rc = check_transformer(source_type, target_type, transformer);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  if (!valid_view(source, source_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (target == nullptr || target_length < 0) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (target_length < source_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (source_stride < 1 || target_stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(source, elem_size(source_type)) ||
+      !aligned_to(target, elem_size(target_type)))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  TransformArgs a{source, source_stride, source_type, target, target_stride,
+                  target_type, nullptr, source_length, transformer, factor};
+  return launch_transform(static_cast<hipStream_t>(stream), a);
+}
+
+int32_t ilgpu_hip_reorder_transform(ilgpu_hip_stream_t stream,
+                                    const void* source, int64_t source_length,
+                                    int32_t source_type, void* target,
+                                    int64_t target_length, int32_t target_type,
+                                    const int32_t* order, int64_t order_length,
+                                    int32_t transformer, int64_t factor) {
+  /* ReorderExtensions.cs:158-171, then TransformExtensions.cs:304-317 with
+   * the order view as the transformer's source. */
+  const int32_t rc = check_transformer(source_type, target_type, transformer);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  if (!valid_view(source, source_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(order, order_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (order_length < source_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (source_length > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(target, target_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (target_length < order_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(source, elem_size(source_type)) ||
+      !aligned_to(target, elem_size(target_type)) || !aligned_to(order, 4))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  TransformArgs a{source, 1, source_type, target, 1, target_type, order,
+                  order_length, transformer, factor};
+  return launch_transform(static_cast<hipStream_t>(stream), a);
+}
+
 }  // extern "C"

@@ -59,6 +59,21 @@ int32_t launch_sequence(hipStream_t stream, void* view, int64_t n, int64_t strid
 int32_t launch_reorder(hipStream_t stream, const void* source, void* target,
                        const int32_t* order, int64_t n, int elem_bytes);
 
+// transform.hip: target[i] = (T)op((S)source[order ? order[i] : i]).
+struct TransformArgs {
+  const void* source;
+  int64_t source_stride;  // ignored when order is given (dense source)
+  int32_t source_type;
+  void* target;
+  int64_t target_stride;
+  int32_t target_type;
+  const int32_t* order;   // nullptr for a plain transform
+  int64_t n;
+  int32_t transformer;
+  int64_t factor;
+};
+int32_t launch_transform(hipStream_t stream, const TransformArgs& args);
+
 // fill kernel shared by scan and sort: words[0..count) = 0, as a kernel so
 // that callers may capture the stream into a graph.
 int32_t launch_zero_words(hipStream_t stream, uint32_t* words, int64_t count);

@@ -828,5 +828,156 @@ void Reorder(Accelerator&, AcceleratorStream& stream, ArrayView<T> source, Array
       "target");
 }
 
+// ---- transform (TransformExtensions.cs:24-55, 73-115, 255-506) -------------------------------
+// The reference accepts any struct implementing ITransformer<TSource, TTarget>; this layer
+// accepts the transformers below, each of the form (TTarget)op((TSource)value) with op closed
+// in the source type.  They cover IdentityTransformer and the transformers of the reference's
+// tests (Generic/AlgorithmsTestData.tt:170-252: IntToLong, UIntToULong, IntToNegInt,
+// UInt32ToBitCompInt32, UInt64ToBitCompInt64, <T>Mul2, Index1To<T>).
+template <typename T>
+struct IdentityTransformer {           // TransformExtensions.cs:42-55
+  using Source = T; using Target = T;
+  static constexpr int32_t Kind = ILGPU_HIP_TRANSFORM_CONVERT;
+  int64_t Factor() const { return 0; }
+};
+template <typename TSource, typename TTarget>
+struct ConvertTransformer {            // value => (TTarget)value
+  using Source = TSource; using Target = TTarget;
+  static constexpr int32_t Kind = ILGPU_HIP_TRANSFORM_CONVERT;
+  int64_t Factor() const { return 0; }
+};
+template <typename TSource, typename TTarget = TSource>
+struct NegateTransformer {             // value => (TTarget)(-value)
+  using Source = TSource; using Target = TTarget;
+  static constexpr int32_t Kind = ILGPU_HIP_TRANSFORM_NEGATE;
+  int64_t Factor() const { return 0; }
+};
+template <typename TSource, typename TTarget = TSource>
+struct BitComplementTransformer {      // value => (TTarget)~value
+  using Source = TSource; using Target = TTarget;
+  static constexpr int32_t Kind = ILGPU_HIP_TRANSFORM_BIT_COMPLEMENT;
+  int64_t Factor() const { return 0; }
+};
+template <typename TSource, typename TTarget = TSource>
+struct MultiplyTransformer {           // value => (TTarget)(value * (TSource)factor)
+  using Source = TSource; using Target = TTarget;
+  static constexpr int32_t Kind = ILGPU_HIP_TRANSFORM_MULTIPLY;
+  int64_t factor = 2;
+  int64_t Factor() const { return factor; }
+};
+
+template <typename TSource, typename TSourceStride, typename TTarget, typename TTargetStride,
+          typename TTransformer>
+using StridedTransformer = std::function<void(AcceleratorStream&, ArrayView1D<TSource, TSourceStride>,
+                                              ArrayView1D<TTarget, TTargetStride>, TTransformer)>;
+template <typename TSource, typename TTarget, typename TTransformer>
+using Transformer = std::function<void(AcceleratorStream&, ArrayView<TSource>, ArrayView<TTarget>,
+                                       TTransformer)>;
+template <typename TSource, typename TTarget, typename TTransformer>
+using ReorderTransformer = std::function<void(AcceleratorStream&, ArrayView<TSource>,
+                                              ArrayView<TTarget>, ArrayView<Index1D>, TTransformer)>;
+
+// CreateTransformer, strided form (TransformExtensions.cs:289-345).
+template <typename TSource, typename TSourceStride, typename TTarget, typename TTargetStride,
+          typename TTransformer>
+StridedTransformer<TSource, TSourceStride, TTarget, TTargetStride, TTransformer>
+CreateTransformer(Accelerator&) {
+  static_assert(std::is_same<typename TTransformer::Source, TSource>::value &&
+                    std::is_same<typename TTransformer::Target, TTarget>::value,
+                "the transformer must map TSource to TTarget");
+  return [](AcceleratorStream& stream, ArrayView1D<TSource, TSourceStride> source,
+            ArrayView1D<TTarget, TTargetStride> target, TTransformer transformer) {
+    if (!source.IsValid()) throw ArgumentNullException("source");
+    if (source.Length() < 1) throw ArgumentOutOfRangeException("source");
+    if (!target.IsValid()) throw ArgumentNullException("source");  // sic, :308-309
+    if (target.Length() < source.Length()) throw ArgumentOutOfRangeException("target");
+    HipAlgorithmsException::ThrowIfFailed(
+        ilgpu_hip_transform(stream.StreamPtr(), source.LoadEffectiveAddressAsPtr(),
+                            source.Length(), source.Stride().Stride(),
+                            TypeCode<TSource>::value, target.LoadEffectiveAddressAsPtr(),
+                            target.Length(), target.Stride().Stride(), TypeCode<TTarget>::value,
+                            TTransformer::Kind, transformer.Factor()),
+        "target");
+  };
+}
+// CreateTransformer, dense form (:255-270).
+template <typename TSource, typename TTarget, typename TTransformer>
+Transformer<TSource, TTarget, TTransformer> CreateTransformer(Accelerator& accelerator) {
+  auto launcher = CreateTransformer<TSource, Stride1D::Dense, TTarget, Stride1D::Dense,
+                                    TTransformer>(accelerator);
+  return [launcher](AcceleratorStream& stream, ArrayView<TSource> source,
+                    ArrayView<TTarget> target, TTransformer transformer) {
+    launcher(stream, ArrayView1D<TSource, Stride1D::Dense>(source),
+             ArrayView1D<TTarget, Stride1D::Dense>(target), transformer);
+  };
+}
+// CreateTransformer<T, TTransformer> (:356-361).
+template <typename T, typename TTransformer>
+Transformer<T, T, TTransformer> CreateTransformer(Accelerator& accelerator) {
+  return CreateTransformer<T, T, TTransformer>(accelerator);
+}
+// Transform, in place (:377-393), source to target (:411-428) and strided (:479-506).
+template <typename T, typename TTransformer>
+void Transform(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<T> view,
+               TTransformer transformer) {
+  CreateTransformer<T, T, TTransformer>(accelerator)(stream, view, view, transformer);
+}
+template <typename TSource, typename TTarget, typename TTransformer>
+void Transform(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<TSource> source,
+               ArrayView<TTarget> target, TTransformer transformer) {
+  CreateTransformer<TSource, TTarget, TTransformer>(accelerator)(stream, source, target,
+                                                                 transformer);
+}
+template <typename TSource, typename TSourceStride, typename TTarget, typename TTargetStride,
+          typename TTransformer>
+void Transform(Accelerator& accelerator, AcceleratorStream& stream,
+               ArrayView1D<TSource, TSourceStride> source,
+               ArrayView1D<TTarget, TTargetStride> target, TTransformer transformer) {
+  CreateTransformer<TSource, TSourceStride, TTarget, TTargetStride, TTransformer>(accelerator)(
+      stream, source, target, transformer);
+}
+
+// CreateReorderTransformer (ReorderExtensions.cs:143-182) and ReorderTransform (:232-297).
+template <typename TSource, typename TTarget, typename TTransformer>
+ReorderTransformer<TSource, TTarget, TTransformer> CreateReorderTransformer(Accelerator&) {
+  static_assert(std::is_same<typename TTransformer::Source, TSource>::value &&
+                    std::is_same<typename TTransformer::Target, TTarget>::value,
+                "the transformer must map TSource to TTarget");
+  return [](AcceleratorStream& stream, ArrayView<TSource> source, ArrayView<TTarget> target,
+            ArrayView<Index1D> reorderView, TTransformer transformer) {
+    if (!source.IsValid()) throw ArgumentNullException("source");
+    if (source.Length() < 1) throw ArgumentOutOfRangeException("source");
+    if (!reorderView.IsValid()) throw ArgumentNullException("reorderView");
+    if (reorderView.Length() < source.Length()) throw ArgumentOutOfRangeException("reorderView");
+    if (source.Length() > std::numeric_limits<int32_t>::max())
+      throw NotSupportedException("NotSupportedArrayView64");
+    if (!target.IsValid()) throw ArgumentNullException("source");  // sic
+    if (target.Length() < reorderView.Length()) throw ArgumentOutOfRangeException("target");
+    HipAlgorithmsException::ThrowIfFailed(
+        ilgpu_hip_reorder_transform(stream.StreamPtr(), source.LoadEffectiveAddressAsPtr(),
+                                    source.Length(), TypeCode<TSource>::value,
+                                    target.LoadEffectiveAddressAsPtr(), target.Length(),
+                                    TypeCode<TTarget>::value,
+                                    reorderView.LoadEffectiveAddressAsPtr(),
+                                    reorderView.Length(), TTransformer::Kind,
+                                    transformer.Factor()),
+        "target");
+  };
+}
+template <typename T, typename TTransformer>
+void ReorderTransform(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<T> source,
+                      ArrayView<T> target, ArrayView<Index1D> reorderView,
+                      TTransformer transformer) {
+  CreateReorderTransformer<T, T, TTransformer>(accelerator)(stream, source, target, reorderView,
+                                                            transformer);
+}
+template <typename TSource, typename TTarget, typename TTransformer>
+void ReorderTransform(Accelerator& accelerator, AcceleratorStream& stream,
+                      ArrayView<TSource> source, ArrayView<TTarget> target,
+                      ArrayView<Index1D> reorderView, TTransformer transformer) {
+  CreateReorderTransformer<TSource, TTarget, TTransformer>(accelerator)(
+      stream, source, target, reorderView, transformer);
+}
+
 }  // namespace Algorithms
 }  // namespace ilgpu

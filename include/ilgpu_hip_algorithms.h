@@ -242,8 +242,6 @@ int32_t ilgpu_hip_unique(ilgpu_hip_stream_t stream, void *input, int64_t n,
  * (ReorderExtensions.cs:194-214): target[i] = source[order[i]] for
  * i < order_length, with the reference's checks order_length >= source_length
  * and target_length >= order_length.  Index values are not range-checked.
- * Transformers with user-written functors are not offered: they need the
- * reference's JIT.
  */
 int32_t ilgpu_hip_initialize(ilgpu_hip_stream_t stream, void *view, int64_t n,
                              int64_t stride, int32_t elem_bytes,
@@ -255,6 +253,48 @@ int32_t ilgpu_hip_reorder(ilgpu_hip_stream_t stream, const void *source,
                           int64_t source_length, void *target,
                           int64_t target_length, const int32_t *order,
                           int64_t order_length, int32_t elem_bytes);
+
+/* ---- transform, reorder-transform ----------------------------------------
+ * Replace: the Transformer delegates, CreateTransformer and Transform
+ * (TransformExtensions.cs:73-115, 255-506): target[i] = f(source[i]) for
+ * i < source_length, with the reference's checks source_length >= 1 and
+ * target_length >= source_length (:304-317); and ReorderTransformer,
+ * CreateReorderTransformer and ReorderTransform (ReorderExtensions.cs:42-52,
+ * 143-297): target[i] = f(source[order[i]]) for i < order_length, with the
+ * checks of ilgpu_hip_reorder.
+ *
+ * The reference JIT-compiles any ITransformer<TSource, TTarget> struct
+ * (TransformExtensions.cs:24-37).  Here the transformers are a closed set of
+ * the form (TTarget)op((TSource)value): op is computed in the source type
+ * (integers wrap, as unchecked C#), then converted to the target type by the
+ * C# explicit numeric conversion (integers truncate or extend by the source's
+ * sign; to and between floating-point types: round to nearest even).  The set
+ * covers IdentityTransformer (:42-55) and every transformer of the reference's
+ * tests (Generic/AlgorithmsTestData.tt:170-252).  Floating-point sources with
+ * integer targets are ILGPU_HIP_ERROR_NOT_SUPPORTED (C# leaves that conversion
+ * unspecified for NaN and out-of-range values), and so is BIT_COMPLEMENT of a
+ * floating-point source.  `factor` is used by MULTIPLY only, converted to the
+ * source type.  A transform with equal source and target types may run in
+ * place (source == target, equal strides).
+ */
+enum ilgpu_hip_transformer {
+  ILGPU_HIP_TRANSFORM_CONVERT = 0,        /* (TTarget)value; identity if the types match */
+  ILGPU_HIP_TRANSFORM_NEGATE = 1,         /* (TTarget)(-value) */
+  ILGPU_HIP_TRANSFORM_BIT_COMPLEMENT = 2, /* (TTarget)(~value), integer sources */
+  ILGPU_HIP_TRANSFORM_MULTIPLY = 3        /* (TTarget)(value * (TSource)factor) */
+};
+int32_t ilgpu_hip_transform(ilgpu_hip_stream_t stream, const void *source,
+                            int64_t source_length, int64_t source_stride,
+                            int32_t source_type, void *target,
+                            int64_t target_length, int64_t target_stride,
+                            int32_t target_type, int32_t transformer,
+                            int64_t factor);
+int32_t ilgpu_hip_reorder_transform(ilgpu_hip_stream_t stream,
+                                    const void *source, int64_t source_length,
+                                    int32_t source_type, void *target,
+                                    int64_t target_length, int32_t target_type,
+                                    const int32_t *order, int64_t order_length,
+                                    int32_t transformer, int64_t factor);
 
 #ifdef __cplusplus
 }

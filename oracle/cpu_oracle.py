@@ -198,6 +198,57 @@ def reorder(source: np.ndarray, order: np.ndarray) -> np.ndarray:
     return np.ascontiguousarray(source)[np.asarray(order, dtype=np.int64)]
 
 
+TRANSFORM_CONVERT, TRANSFORM_NEGATE, TRANSFORM_BIT_COMPLEMENT, TRANSFORM_MULTIPLY = 0, 1, 2, 3
+
+
+def transform(source: np.ndarray, target_dtype, transformer: int = TRANSFORM_CONVERT,
+              factor: int = 0) -> np.ndarray:
+    """TransformImplementation.Execute (TransformExtensions.cs:153-159) for the
+    closed transformer set (TTarget)op((TSource)value): op in the source type
+    (unchecked C#: integers wrap), then the explicit numeric conversion
+    (integers truncate or extend by the source's sign; floating-point targets
+    round to nearest even).  Covers IdentityTransformer (:42-55) and the test
+    transformers of Generic/AlgorithmsTestData.tt:170-252."""
+    src = np.ascontiguousarray(source)
+    sdt, tdt = src.dtype, np.dtype(target_dtype)
+    if sdt.kind == "f" and tdt.kind != "f":
+        raise ValueError("floating point -> integer is unspecified in C#")
+    with np.errstate(over="ignore"):
+        if transformer == TRANSFORM_CONVERT:
+            v = src
+        elif transformer == TRANSFORM_NEGATE:
+            v = -src if sdt.kind == "f" else (0 - src.astype(sdt)).astype(sdt)
+        elif transformer == TRANSFORM_BIT_COMPLEMENT:
+            if sdt.kind == "f":
+                raise ValueError("~ of a floating-point value")
+            v = ~src
+        elif transformer == TRANSFORM_MULTIPLY:
+            if sdt.kind == "f":
+                v = src * sdt.type(factor)
+            else:
+                bits = sdt.itemsize * 8
+                k = np.uint64(factor & ((1 << 64) - 1))
+                wide = src.astype(np.int64).view(np.uint64) * k
+                v = (wide & np.uint64((1 << bits) - 1)).astype(
+                    np.dtype("u%d" % sdt.itemsize)).view(sdt)
+        else:
+            raise ValueError(transformer)
+        v = np.asarray(v, dtype=sdt)
+        if sdt.kind != "f" and tdt.kind != "f":
+            wide = v.astype(np.int64 if sdt.kind == "i" else np.uint64).view(np.uint64)
+            tbits = tdt.itemsize * 8
+            mask = np.uint64((1 << tbits) - 1)
+            return (wide & mask).astype(np.dtype("u%d" % tdt.itemsize)).view(tdt)
+        return v.astype(tdt)
+
+
+def reorder_transform(source: np.ndarray, order: np.ndarray, target_dtype,
+                      transformer: int = TRANSFORM_CONVERT, factor: int = 0) -> np.ndarray:
+    """ReorderTransformWrapper.Transform (ReorderExtensions.cs:91-95):
+    target[i] = transformer(source[reorderView[i]])."""
+    return transform(reorder(source, order), target_dtype, transformer, factor)
+
+
 def scan_temp_ints_cpu() -> int:
     return int(lib().oracle_scan_temp_ints_cpu())
 

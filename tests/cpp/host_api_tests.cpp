@@ -364,6 +364,90 @@ template <typename T> void InitializeAndReorderTests(Accelerator& accl) {
   }
 }
 
+// ---- TransformerExtensionTests, ReorderExtensionTests (transformers) ---------------
+// TransformerExtensionTests.tt:66-134 with the closed-set stand-ins for
+// IntToNegIntTransformer, IntToLongTransformer and UInt32ToBitCompInt32Transformer.
+void TransformTests(Accelerator& accl) {
+  auto& s = accl.DefaultStream();
+  for (int length : kArraySizes) {
+    const auto seq = ComputeSequence<int32_t>(42, 0, length);
+    auto input = accl.Allocate1D<int32_t>(seq);
+    auto output = accl.Allocate1D<int32_t>(length);
+    Transform<int32_t, int32_t>(accl, s, input->View(), output->View(),
+                                NegateTransformer<int32_t>());
+    accl.Synchronize();
+    CHECK(Verify(output->GetAsArray1D(), std::vector<int32_t>((size_t)length, -42)));
+
+    auto wide = accl.Allocate1D<int64_t>(length);
+    auto transformer = CreateTransformer<int32_t, int64_t, ConvertTransformer<int32_t, int64_t>>(accl);
+    transformer(s, input->View(), wide->View(), ConvertTransformer<int32_t, int64_t>());
+    accl.Synchronize();
+    CHECK(Verify(wide->GetAsArray1D(), std::vector<int64_t>((size_t)length, 42)));
+
+    const auto useq = ComputeSequence<uint32_t>(0, 1, length);
+    auto uinput = accl.Allocate1D<uint32_t>(useq);
+    Transform<uint32_t, int32_t>(accl, s, uinput->View(), output->View(),
+                                 BitComplementTransformer<uint32_t, int32_t>());
+    accl.Synchronize();
+    std::vector<int32_t> comp((size_t)length);
+    for (int i = 0; i < length; ++i) comp[i] = (int32_t)~useq[i];
+    CHECK(Verify(output->GetAsArray1D(), comp));
+
+    // in place (TransformExtensions.cs:377-393)
+    Transform<int32_t>(accl, s, input->View(), MultiplyTransformer<int32_t>{3});
+    accl.Synchronize();
+    CHECK(Verify(input->GetAsArray1D(), std::vector<int32_t>((size_t)length, 126)));
+
+    if (length > 1) {
+      EXPECT_THROW((Transform<int32_t, int32_t>(accl, s, input->View(),
+                                                 output->View().SubView(0, length - 1),
+                                                 NegateTransformer<int32_t>())),
+                   ArgumentOutOfRangeException);
+    }
+    EXPECT_THROW((Transform<int32_t, int32_t>(accl, s, ArrayView<int32_t>(), output->View(),
+                                               NegateTransformer<int32_t>())),
+                 ArgumentNullException);
+  }
+}
+
+// TransformerExtensionTests.tt:136-162: Index1D -> T.
+template <typename T> void CastFromIndexTests(Accelerator& accl) {
+  for (int length : kArraySizes) {
+    const auto seq = ComputeSequence<Index1D>(0, 1, length);
+    auto input = accl.Allocate1D<Index1D>(seq);
+    auto output = accl.Allocate1D<T>(length);
+    Transform<Index1D, T>(accl, accl.DefaultStream(), input->View(), output->View(),
+                          ConvertTransformer<Index1D, T>());
+    accl.Synchronize();
+    std::vector<T> expected((size_t)length);
+    for (int i = 0; i < length; ++i) expected[i] = (T)seq[i];
+    CHECK(Verify(output->GetAsArray1D(), expected));
+  }
+}
+
+// ReorderExtensionTests.tt:160-200 (<T>Mul2, reversed order) and :240-290 (widening).
+template <typename T> void ReorderTransformTests(Accelerator& accl) {
+  auto& s = accl.DefaultStream();
+  for (int length : kArraySizes) {
+    for (int variant = 0; variant < 3; ++variant) {
+      const auto seq = variant == 0 ? ComputeSequence<T>(0, 0, length)
+                     : variant == 1 ? ComputeSequence<T>(1, 0, length)
+                                    : ComputeSequence<T>(0, 1, length);
+      std::vector<Index1D> rev((size_t)length);
+      for (int i = 0; i < length; ++i) rev[i] = length - 1 - i;
+      auto input = accl.Allocate1D<T>(seq);
+      auto order = accl.Allocate1D<Index1D>(rev);
+      auto output = accl.Allocate1D<T>(length);
+      ReorderTransform<T>(accl, s, input->View(), output->View(), order->View(),
+                          MultiplyTransformer<T>{2});
+      accl.Synchronize();
+      std::vector<T> expected((size_t)length);   // CalcValues: result[order[i]] = f(input[i])
+      for (int i = 0; i < length; ++i) expected[rev[i]] = (T)(seq[i] * 2);
+      CHECK(Verify(output->GetAsArray1D(), expected));
+    }
+  }
+}
+
 // ---- ReductionExtensionTests ----------------------------------------------------
 template <typename T, typename TOp> void ReduceTests(Accelerator& accl, int maxLength) {
   for (int length : kArraySizes) {
@@ -517,6 +601,16 @@ int main(int argc, char** argv) {
     RUN(InitializeAndReorderTests<int32_t>(accl));
     RUN(InitializeAndReorderTests<uint16_t>(accl));
     RUN(InitializeAndReorderTests<double>(accl));
+    RUN(TransformTests(accl));
+    RUN(CastFromIndexTests<int32_t>(accl));
+    RUN(CastFromIndexTests<int64_t>(accl));
+    RUN(CastFromIndexTests<uint32_t>(accl));
+    RUN(CastFromIndexTests<uint64_t>(accl));
+    RUN(CastFromIndexTests<float>(accl));
+    RUN(CastFromIndexTests<double>(accl));
+    RUN(ReorderTransformTests<int32_t>(accl));
+    RUN(ReorderTransformTests<uint64_t>(accl));
+    RUN(ReorderTransformTests<float>(accl));
   }
   std::printf("%d test groups, %d failed checks\n", g_run, g_failed);
   return g_failed == 0 ? 0 : 1;

@@ -165,3 +165,32 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(capi, "LIB_PATH", "/nonexistent/libilgpu_hip_algorithms.so")
     with pytest.raises(FileNotFoundError):
         capi.lib()
+
+
+def test_transform_argument_validation():
+    L = capi.lib()
+
+    def call(src=FAKE, n=16, s_in=1, st=capi.I32, dst=FAKE, n_out=16, s_out=1, tt=capi.I64,
+             op=capi.TRANSFORM_CONVERT):
+        return L.ilgpu_hip_transform(None, src, n, s_in, st, dst, n_out, s_out, tt, op, 0)
+
+    assert call(src=None) == capi.ERROR_NULL_VIEW          # TransformExtensions.cs:304-305
+    assert call(dst=None) == capi.ERROR_NULL_VIEW          # :308-309
+    assert call(n_out=8) == capi.ERROR_OUT_OF_RANGE        # :310-317
+    assert call(s_in=0) == capi.ERROR_OUT_OF_RANGE
+    assert call(s_out=-1) == capi.ERROR_OUT_OF_RANGE
+    assert call(st=99) == capi.ERROR_NOT_SUPPORTED
+    assert call(op=7) == capi.ERROR_NOT_SUPPORTED
+    assert call(st=capi.F32, tt=capi.I32) == capi.ERROR_NOT_SUPPORTED
+    assert call(st=capi.F64, tt=capi.F64, op=capi.TRANSFORM_BIT_COMPLEMENT) == capi.ERROR_NOT_SUPPORTED
+
+    def rcall(src=FAKE, n=16, dst=FAKE, n_out=16, order=FAKE, n_order=16, st=capi.U32, tt=capi.U32):
+        return L.ilgpu_hip_reorder_transform(None, src, n, st, dst, n_out, tt, order, n_order,
+                                             capi.TRANSFORM_MULTIPLY, 2)
+
+    assert rcall(src=None) == capi.ERROR_NULL_VIEW         # ReorderExtensions.cs:158-159
+    assert rcall(order=None) == capi.ERROR_NULL_VIEW       # :162-163
+    assert rcall(n_order=8) == capi.ERROR_OUT_OF_RANGE     # :164-165
+    assert rcall(n_out=8) == capi.ERROR_OUT_OF_RANGE
+    assert rcall(n=(1 << 31), n_order=(1 << 31), n_out=(1 << 31)) == capi.ERROR_NOT_SUPPORTED  # :166-170
+    assert rcall(st=capi.F16, tt=capi.U8) == capi.ERROR_NOT_SUPPORTED

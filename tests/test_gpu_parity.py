@@ -736,6 +736,129 @@ def test_reorder(dtype):
         capi.reorder(D.zeros(10, dtype), D.zeros(9, dtype), D.zeros(10, np.int32))
 
 
+ALL_NUMERIC = [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64,
+               np.uint64, np.float16, np.float32, np.float64]
+
+
+def _transform_input(dtype, n, seed):
+    dt = np.dtype(dtype)
+    if dt.kind == "f":
+        # finite values of every magnitude the type holds, both signs, zeros, and
+        # specials; doubles include values that fall between float16/float32 neighbours
+        r = np.random.default_rng(seed)
+        mag = np.exp(r.uniform(-40, 40, n)) if dt.itemsize > 2 else np.exp(r.uniform(-12, 11, n))
+        v = (mag * r.choice([-1.0, 1.0], n)).astype(dt)
+        v[:8] = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 65519.99], dtype=dt)[: min(8, n)]
+        if dt.itemsize == 8 and n > 12:
+            # just above the midpoint of two float16 neighbours: rounding to float32 first
+            # would land on the midpoint and then round the wrong way
+            v[8:12] = [1 + 2.0 ** -11 + 2.0 ** -40, -(1 + 2.0 ** -11 + 2.0 ** -40),
+                       1 + 3 * 2.0 ** -11 - 2.0 ** -40, 2.0 ** -25 + 2.0 ** -60]
+        return v
+    v = random_ints(dtype, n, seed=seed)
+    info = np.iinfo(dtype)
+    edge = np.array([0, 1, info.max, info.min, info.max - 1], dtype=dtype)
+    v[: min(5, n)] = edge[: min(5, n)]
+    return v
+
+
+def _same_bits(a, b):
+    if a.dtype.kind == "f":   # NaN payloads are not pinned: compare NaN-ness, then the rest bitwise
+        na, nb = np.isnan(a), np.isnan(b)
+        return np.array_equal(na, nb) and np.array_equal(a[~na].view(np.uint8), b[~nb].view(np.uint8))
+    return np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("sdt", ALL_NUMERIC)
+def test_transform_every_type_pair_and_transformer(sdt):
+    n = 5000
+    src = _transform_input(sdt, n, seed=np.dtype(sdt).num)
+    d_src = D.from_numpy(src)
+    for tdt in ALL_NUMERIC:
+        if np.dtype(sdt).kind == "f" and np.dtype(tdt).kind != "f":
+            with pytest.raises(capi.NotSupportedError):
+                capi.transform(d_src, D.zeros(n, tdt))
+            continue
+        for op, factor in ((capi.TRANSFORM_CONVERT, 0), (capi.TRANSFORM_NEGATE, 0),
+                           (capi.TRANSFORM_BIT_COMPLEMENT, 0), (capi.TRANSFORM_MULTIPLY, 2),
+                           (capi.TRANSFORM_MULTIPLY, -3)):
+            if op == capi.TRANSFORM_BIT_COMPLEMENT and np.dtype(sdt).kind == "f":
+                continue
+            note("transform", np.dtype(sdt).name, np.dtype(tdt).name, op, factor)
+            tgt = D.zeros(n, tdt)
+            capi.transform(d_src, tgt, op, factor)
+            sync()
+            assert _same_bits(tgt.numpy(), O.transform(src, tdt, op, factor)), (sdt, tdt, op)
+
+
+@pytest.mark.parametrize("n", ARRAY_SIZES + [1 << 20, (1 << 20) + 3])
+def test_transform_reference_cases(n):
+    # TransformerExtensionTests.tt:66-134
+    seq = compute_sequence(np.int32, 42, 0, n)
+    out = D.zeros(n, np.int32)
+    capi.transform(D.from_numpy(seq), out, capi.TRANSFORM_NEGATE)
+    out64 = D.zeros(n, np.int64)
+    capi.transform(D.from_numpy(seq), out64)
+    useq = compute_sequence(np.uint32, 0, 1, n)
+    comp = D.zeros(n, np.int32)
+    capi.transform(D.from_numpy(useq), comp, capi.TRANSFORM_BIT_COMPLEMENT)
+    sync()
+    assert np.array_equal(out.numpy(), np.full(n, -42, dtype=np.int32))
+    assert np.array_equal(out64.numpy(), np.full(n, 42, dtype=np.int64))
+    assert np.array_equal(comp.numpy(), (-1 - np.arange(n)).astype(np.int32))
+
+
+def test_transform_in_place_strided_and_longer_target():
+    n = 10007
+    src = random_ints(np.int32, n, seed=9)
+    d = D.from_numpy(src)
+    capi.transform(d, d, capi.TRANSFORM_NEGATE)      # in place
+    sync()
+    assert np.array_equal(d.numpy(), O.transform(src, np.int32, O.TRANSFORM_NEGATE))
+    # strided source and target views; elements between the strides stay untouched
+    base = random_ints(np.int16, 3 * n, seed=10)
+    out = np.full(2 * n + 5, 77, dtype=np.int64)
+    d_base_in, d_base_out = D.from_numpy(base), D.from_numpy(out)
+    d_in, d_out = d_base_in.strided(3), d_base_out.strided(2)
+    assert d_in.length == n and d_out.length >= n
+    capi.transform(d_in, d_out, capi.TRANSFORM_MULTIPLY, 2)
+    sync()
+    expect = out.copy()
+    expect[0: 2 * n: 2] = O.transform(base[::3], np.int64, O.TRANSFORM_MULTIPLY, 2)
+    assert np.array_equal(d_base_out.numpy(), expect)
+    # TransformExtensions.cs:310-317: a short target is refused
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.transform(D.zeros(10, np.int32), D.zeros(9, np.int32))
+
+
+@pytest.mark.parametrize("dtype", ATOMIC_NUMERIC_DTYPES)
+def test_reorder_transform_reference_case_and_random_gather(dtype):
+    # ReorderExtensionTests.tt:160-200: reversed order, value * 2
+    for n in ARRAY_SIZES:
+        for start, step in ((0, 0), (1, 0), (0, 1)):
+            seq = compute_sequence(dtype, start, step, n)
+            order = np.arange(n - 1, -1, -1, dtype=np.int32)
+            tgt = D.zeros(n, dtype)
+            capi.reorder_transform(D.from_numpy(seq), tgt, D.from_numpy(order),
+                                   capi.TRANSFORM_MULTIPLY, 2)
+            sync()
+            with np.errstate(over="ignore"):
+                expect = (seq + seq)[::-1]
+            assert np.array_equal(tgt.numpy().view(np.uint8), np.ascontiguousarray(expect).view(np.uint8))
+    # ReorderExtensionTests.tt:69-112: widening and bit-complement transformers, random order
+    n = 1 << 18
+    for sdt, tdt, op in ((np.int32, np.int64, capi.TRANSFORM_CONVERT),
+                         (np.uint32, np.uint64, capi.TRANSFORM_CONVERT),
+                         (np.uint32, np.int32, capi.TRANSFORM_BIT_COMPLEMENT),
+                         (np.uint64, np.int64, capi.TRANSFORM_BIT_COMPLEMENT)):
+        src = random_ints(sdt, n, seed=21)
+        order = np.random.default_rng(22).permutation(n).astype(np.int32)
+        tgt = D.zeros(n, tdt)
+        capi.reorder_transform(D.from_numpy(src), tgt, D.from_numpy(order), op)
+        sync()
+        assert np.array_equal(tgt.numpy(), O.reorder_transform(src, order, tdt, op))
+
+
 def test_sort_then_unique_pipeline():
     # the pipeline the two primitives are used for: distinct keys of a column
     keys = datagen.zipf_u32(1 << 22)

@@ -405,3 +405,107 @@ def test_reorder_is_a_gather():
     out = O.reorder(src, order)
     for i in range(50):
         assert out[i] == src[order[i]]
+
+
+# ------------------------------------------------------------------ transform
+def _py_convert(values, sdt, tdt):
+    """Integer conversion by Python big-int arithmetic: value mod 2^bits, read
+    back in the target's signedness."""
+    bits = np.dtype(tdt).itemsize * 8
+    out = []
+    for v in values:
+        w = int(v) % (1 << bits)
+        if np.dtype(tdt).kind == "i" and w >= 1 << (bits - 1):
+            w -= 1 << bits
+        out.append(w)
+    return np.array(out, dtype=tdt)
+
+
+@pytest.mark.parametrize("n", ARRAY_SIZES)
+def test_transform_reference_cases(n):
+    # TransformerExtensionTests.tt:66-86: 42, 42, ... -> -42.
+    seq = compute_sequence(np.int32, 42, 0, n)
+    assert np.array_equal(O.transform(seq, np.int32, O.TRANSFORM_NEGATE),
+                          np.full(n, -42, dtype=np.int32))
+    # :88-111: (long)x.
+    got = O.transform(seq, np.int64)
+    assert got.dtype == np.int64 and np.array_equal(got, np.full(n, 42, dtype=np.int64))
+    # :113-134: (int)~x for x = 0, 1, 2, ... is -1 - x.
+    useq = compute_sequence(np.uint32, 0, 1, n)
+    assert np.array_equal(O.transform(useq, np.int32, O.TRANSFORM_BIT_COMPLEMENT),
+                          (-1 - np.arange(n)).astype(np.int32))
+
+
+@pytest.mark.parametrize("dtype", ATOMIC_NUMERIC_DTYPES)
+@pytest.mark.parametrize("n", ARRAY_SIZES)
+def test_transform_cast_from_index_reference_case(dtype, n):
+    # TransformerExtensionTests.tt:136-162 with Index1To<T>Transformer
+    # (AlgorithmsTestData.tt:239-252): index i -> (T)i.
+    idx = compute_sequence(np.int32, 0, 1, n)
+    got = O.transform(idx, dtype)
+    assert got.dtype == np.dtype(dtype)
+    assert [float(x) for x in got] == [float(i) for i in range(n)]
+
+
+@pytest.mark.parametrize("dtype", ATOMIC_NUMERIC_DTYPES)
+@pytest.mark.parametrize("start,step", [(0, 0), (1, 0), (0, 1), (-1, 0), (0, -1)])
+def test_reorder_transform_mul2_reverse_reference_case(dtype, start, step):
+    # ReorderExtensionTests.tt:43-66, 160-200: reversed order, value * 2;
+    # expectation built the reference's way, result[order[i]] = 2 * input[i].
+    if np.dtype(dtype).kind == "u" and (start < 0 or step < 0):
+        pytest.skip("the reference skips negative sequences for unsigned types")
+    for n in ARRAY_SIZES:
+        seq = compute_sequence(dtype, start, step, n)
+        order = np.arange(n - 1, -1, -1, dtype=np.int32)
+        expect = np.empty(n, dtype=dtype)
+        with np.errstate(over="ignore"):
+            for i in range(n):
+                expect[order[i]] = seq[i] + seq[i]
+        got = O.reorder_transform(seq, order, dtype, O.TRANSFORM_MULTIPLY, 2)
+        assert np.array_equal(got.view(np.uint8), expect.view(np.uint8))
+
+
+@pytest.mark.parametrize("sdt", INT_KEY_DTYPES)
+@pytest.mark.parametrize("tdt", INT_KEY_DTYPES)
+def test_transform_integer_semantics_by_big_int_arithmetic(sdt, tdt):
+    info = np.iinfo(sdt)
+    edge = np.array([0, 1, info.max, info.min, info.max - 1, info.min + 1 if info.min else 2],
+                    dtype=sdt)
+    vals = np.concatenate([edge, random_ints(sdt, 200, seed=5)])
+    sbits = np.dtype(sdt).itemsize * 8
+
+    def in_source(py_values):   # wrap to the source type first (op is closed in it)
+        return _py_convert(py_values, sdt, sdt)
+
+    assert np.array_equal(O.transform(vals, tdt), _py_convert(vals, sdt, tdt))
+    neg = in_source([-int(v) for v in vals])
+    assert np.array_equal(O.transform(vals, tdt, O.TRANSFORM_NEGATE), _py_convert(neg, sdt, tdt))
+    comp = in_source([-1 - int(v) for v in vals])   # ~v = -1 - v
+    assert np.array_equal(O.transform(vals, tdt, O.TRANSFORM_BIT_COMPLEMENT),
+                          _py_convert(comp, sdt, tdt))
+    for k in (2, -3, 1 << 40):
+        mul = in_source([int(v) * k for v in vals])
+        assert np.array_equal(O.transform(vals, tdt, O.TRANSFORM_MULTIPLY, k),
+                              _py_convert(mul, sdt, tdt))
+    assert sbits in (8, 16, 32, 64)
+
+
+def test_transform_float_semantics():
+    x = np.array([0.0, -0.0, 1.5, -2.25, 65519.0, 65520.0, 1e-8, np.inf, -np.inf, np.nan],
+                 dtype=np.float64)
+    h = O.transform(x, np.float16)
+    assert h[4] == 65504 and h[5] == np.inf and h[6] == 0 and np.isnan(h[9])   # RNE, overflow, underflow
+    assert np.signbit(O.transform(x, np.float32, O.TRANSFORM_NEGATE)[0])        # -(+0) = -0
+    # one rounding, not two: just above a float16 midpoint goes up
+    above = np.array([1 + 2.0 ** -11 + 2.0 ** -40], dtype=np.float64)
+    assert float(O.transform(above, np.float16)[0]) == 1 + 2.0 ** -10
+    assert np.array_equal(O.transform(x[2:4], np.float64, O.TRANSFORM_MULTIPLY, 2), [3.0, -4.5])
+    # integer -> float rounds to nearest even: 2^24 + 1 -> 2^24, 2^24 + 3 -> 2^24 + 4
+    i = np.array([(1 << 24) + 1, (1 << 24) + 3, -(1 << 24) - 1], dtype=np.int32)
+    assert [float(v) for v in O.transform(i, np.float32)] == [16777216.0, 16777220.0, -16777216.0]
+    u = np.array([(1 << 64) - 1, (1 << 53) + 1], dtype=np.uint64)
+    assert [float(v) for v in O.transform(u, np.float64)] == [float(1 << 64), float(1 << 53)]
+    with pytest.raises(ValueError):
+        O.transform(x, np.int32)
+    with pytest.raises(ValueError):
+        O.transform(x, np.float64, O.TRANSFORM_BIT_COMPLEMENT)
