@@ -85,12 +85,53 @@ __global__ __launch_bounds__(kBlock) void transform_kernel(
   }
 }
 
+// Dense views: K consecutive elements per thread, K chosen so that the wider
+// of the two element types moves as one 16-byte vector.  The last n % K
+// elements go through the scalar kernel.
+template <typename E, int K> struct alignas(sizeof(E) * K) Pack { E v[K]; };
+
+template <typename S, typename T, int K>
+__global__ __launch_bounds__(kBlock) void transform_dense_kernel(
+    const Pack<S, K>* source, Pack<T, K>* target, int64_t packs, int op, int64_t factor) {
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < packs; i += step) {
+    const Pack<S, K> in = source[i];
+    Pack<T, K> out;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      out.v[k] = convert<S, T>(apply_transformer<S>(in.v[k], op, factor));
+    target[i] = out;
+  }
+}
+
 template <typename S, typename T>
 int32_t transform_typed(hipStream_t stream, const TransformArgs& a) {
   if constexpr (is_float_type<S>::value && !is_float_type<T>::value) {
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   } else {
     ProfileScope scope(stream, a.order != nullptr ? "reorder_transform" : "transform");
+    constexpr int kWide = sizeof(S) > sizeof(T) ? sizeof(S) : sizeof(T);
+    constexpr int K = 16 / kWide;
+    const bool dense = a.order == nullptr && a.source_stride == 1 && a.target_stride == 1 &&
+                       reinterpret_cast<uintptr_t>(a.source) % (sizeof(S) * K) == 0 &&
+                       reinterpret_cast<uintptr_t>(a.target) % (sizeof(T) * K) == 0;
+    if (K > 1 && dense && a.n >= K) {
+      const int64_t packs = a.n / K;
+      hipLaunchKernelGGL((transform_dense_kernel<S, T, K>), dim3((unsigned)grid_for(packs)),
+                         dim3(kBlock), 0, stream,
+                         static_cast<const Pack<S, K>*>(a.source),
+                         static_cast<Pack<T, K>*>(a.target), packs, a.transformer, a.factor);
+      ILGPU_HIP_CHECK(hipGetLastError());
+      const int64_t done = packs * K;
+      if (done == a.n) return ILGPU_HIP_SUCCESS;
+      hipLaunchKernelGGL((transform_kernel<S, T>), dim3(1), dim3(kBlock), 0, stream,
+                         static_cast<const S*>(a.source) + done, (int64_t)1,
+                         static_cast<T*>(a.target) + done, (int64_t)1,
+                         static_cast<const int32_t*>(nullptr), a.n - done, a.transformer,
+                         a.factor);
+      ILGPU_HIP_CHECK(hipGetLastError());
+      return ILGPU_HIP_SUCCESS;
+    }
     hipLaunchKernelGGL((transform_kernel<S, T>), dim3((unsigned)grid_for(a.n)),
                        dim3(kBlock), 0, stream, static_cast<const S*>(a.source),
                        a.source_stride, static_cast<T*>(a.target), a.target_stride,

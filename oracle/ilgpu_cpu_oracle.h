@@ -30,6 +30,11 @@
  *                               only (no reference test has such inputs).
  *   sequence / initialize / reorder (numpy restatements in cpu_oracle.py) pinned by
  *                               SequencerTests.tt:56-70 and ReorderExtensionTests.tt.
+ *   transform / reorder_transform (numpy restatements in cpu_oracle.py) pinned by the
+ *                               expectations of TransformerExtensionTests.tt:66-162
+ *                               and ReorderExtensionTests.tt:160-290, and by Python
+ *                               big-integer arithmetic for every integer type pair;
+ *                               float16/32/64 rounding by hand-picked ties.
  *   temp-size helpers           pinned by the closed formulas they restate.
  */
 #ifndef ILGPU_CPU_ORACLE_H

@@ -831,6 +831,25 @@ def test_transform_in_place_strided_and_longer_target():
         capi.transform(D.zeros(10, np.int32), D.zeros(9, np.int32))
 
 
+@pytest.mark.parametrize("sdt,tdt", [(np.int32, np.int32), (np.uint8, np.uint8), (np.int32, np.int64),
+                                     (np.uint8, np.uint64), (np.int64, np.int16), (np.float64, np.float16),
+                                     (np.int16, np.float32)])
+def test_transform_dense_vector_path_heads_and_tails(sdt, tdt):
+    # the dense path moves 16-byte vectors: lengths around whole vectors, and views
+    # that start off a vector boundary (which take the element-wise path)
+    src = _transform_input(sdt, 70000, seed=31)
+    d_src = D.from_numpy(src)
+    for off_in, off_out, n in [(0, 0, 65536), (0, 0, 65537), (0, 0, 65551), (0, 0, 1), (0, 0, 15),
+                               (1, 0, 40000), (0, 3, 40001), (5, 5, 4099), (16, 16, 8191)]:
+        base = np.full(n + off_out + 4, 77, dtype=tdt)
+        d_out = D.from_numpy(base)
+        capi.transform(d_src.subview(off_in, n), d_out.subview(off_out, n), capi.TRANSFORM_MULTIPLY, 3)
+        sync()
+        expect = base.copy()
+        expect[off_out:off_out + n] = O.transform(src[off_in:off_in + n], tdt, O.TRANSFORM_MULTIPLY, 3)
+        assert _same_bits(d_out.numpy(), expect), (sdt, tdt, off_in, off_out, n)
+
+
 @pytest.mark.parametrize("dtype", ATOMIC_NUMERIC_DTYPES)
 def test_reorder_transform_reference_case_and_random_gather(dtype):
     # ReorderExtensionTests.tt:160-200: reversed order, value * 2
