@@ -1,0 +1,113 @@
+"""Writes tests/golden/known_answers.json: inputs and expected outputs of the
+known-answer cases that the reference's own tests and sample programs define.
+
+The reference (ILGPU.Algorithms) ships no golden files: every expectation is
+computed inside its tests from a closed form.  This script restates those
+closed forms with Python integers (no numpy arithmetic, no oracle, no HIP
+library), so the vectors are independent of everything they are used to check:
+
+  sort      RadixSortExtensionTests.tt:37-131: inverted sequence -> sequence;
+            Samples/AlgorithmsRadixSort/Program.cs:59-63: 32 reversed ints
+  pairs     RadixSortExtensionTests.tt:346-364: values == keys
+  scan      ScanExtensionTests.tt:43-104, 286-305: x_i = start + i*step;
+            Samples/AlgorithmsScan/Program.cs:32-33: 32 twos
+  reduce    ReductionExtensionTests.tt:41-106; Samples/AlgorithmsReduce/Program.cs:29-31
+  histogram HistogramTests.tt:42-103 (1..1024 into 64 / 256 bins by v % bins)
+            and the overflow case :149-189
+  transform TransformerExtensionTests.tt:66-134
+
+Run from the repository root:  python tests/golden/make_known_answers.py
+"""
+import json
+import os
+
+SIZES = [1, 31, 33, 127, 1027]
+INT_TYPES = {"int32": (32, True), "int64": (64, True), "uint32": (32, False), "uint64": (64, False)}
+
+
+def wrap(v, bits, signed):
+    v %= 1 << bits
+    if signed and v >= 1 << (bits - 1):
+        v -= 1 << bits
+    return v
+
+
+def sequence(start, step, n, bits, signed):
+    return [wrap(start + i * step, bits, signed) for i in range(n)]
+
+
+def main():
+    cases = []
+    for name, (bits, signed) in INT_TYPES.items():
+        for n in SIZES:
+            asc = sequence(0, 1, n, bits, signed)
+            cases.append({"op": "sort", "dtype": name, "descending": False,
+                          "input": asc[::-1], "expected": asc})
+            if n > 127:   # the long cases once per type; the file stays small
+                x = sequence(0, 1, n, bits, signed)
+                cases.append({"op": "scan", "dtype": name, "kind": "inclusive", "scan_op": "add",
+                              "input": x,
+                              "expected": [wrap((i + 1) * i // 2, bits, signed) for i in range(n)]})
+                continue
+            cases.append({"op": "sort", "dtype": name, "descending": True,
+                          "input": asc, "expected": asc[::-1]})
+            cases.append({"op": "sort_pairs", "dtype": name, "input": asc[::-1],
+                          "values": asc[::-1], "expected": asc, "expected_values": asc})
+            for start, step in ((0, 1), (1, 0)) + (((-1, 0), (0, -1)) if signed else ()):
+                x = sequence(start, step, n, bits, signed)
+                inc, acc = [], 0
+                for v in x:
+                    acc = wrap(acc + v, bits, signed)
+                    inc.append(acc)
+                cases.append({"op": "scan", "dtype": name, "kind": "inclusive", "scan_op": "add",
+                              "input": x, "expected": inc})
+                cases.append({"op": "scan", "dtype": name, "kind": "exclusive", "scan_op": "add",
+                              "input": x, "expected": [0] + inc[:-1]})
+                run_max = [max(x[: i + 1]) for i in range(n)]
+                cases.append({"op": "scan", "dtype": name, "kind": "inclusive", "scan_op": "max",
+                              "input": x, "expected": run_max})
+                cases.append({"op": "reduce", "dtype": name, "reduce_op": "add", "input": x,
+                              "expected": inc[-1]})
+                cases.append({"op": "reduce", "dtype": name, "reduce_op": "max", "input": x,
+                              "expected": max(x)})
+                cases.append({"op": "reduce", "dtype": name, "reduce_op": "min", "input": x,
+                              "expected": min(x)})
+    # sample programs
+    rev = list(range(31, -1, -1))
+    cases.append({"op": "sort", "dtype": "int32", "descending": False, "input": rev,
+                  "expected": sorted(rev)})
+    cases.append({"op": "scan", "dtype": "int32", "kind": "inclusive", "scan_op": "add",
+                  "input": [2] * 32, "expected": [2 * (i + 1) for i in range(32)]})
+    cases.append({"op": "scan", "dtype": "int32", "kind": "exclusive", "scan_op": "add",
+                  "input": [2] * 32, "expected": [2 * i for i in range(32)]})
+    cases.append({"op": "reduce", "dtype": "int32", "reduce_op": "add", "input": list(range(64)),
+                  "expected": 2016})
+    # histogram: 1..1024 by v % bins; overflow: bins[0] = max - 33, then 32 samples twice
+    for bins in (64, 256):
+        cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "int32", "locator": "modulo",
+                      "input": list(range(1, 1025)), "bins_before": [0] * bins,
+                      "expected": [1024 // bins] * bins, "expected_overflow": 0})
+    imax = (1 << 31) - 1
+    cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "int32", "locator": "modulo",
+                  "input": [0] * 32, "bins_before": [imax - 33, 0], "expected": [imax - 1, 0],
+                  "expected_overflow": 0})
+    cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "int32", "locator": "modulo",
+                  "input": [0] * 32, "bins_before": [imax - 1, 0],
+                  "expected": [wrap(imax - 1 + 32, 32, True), 0], "expected_overflow": 1})
+    # transform
+    for n in SIZES:
+        cases.append({"op": "transform", "dtype": "int32", "target_dtype": "int32",
+                      "transformer": "negate", "input": [42] * n, "expected": [-42] * n})
+        cases.append({"op": "transform", "dtype": "int32", "target_dtype": "int64",
+                      "transformer": "convert", "input": [42] * n, "expected": [42] * n})
+        cases.append({"op": "transform", "dtype": "uint32", "target_dtype": "int32",
+                      "transformer": "bit_complement", "input": list(range(n)),
+                      "expected": [-1 - i for i in range(n)]})
+    out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "known_answers.json")
+    with open(out, "w") as f:
+        json.dump({"cases": cases}, f, separators=(",", ":"))
+    print(out, len(cases), "cases", os.path.getsize(out), "bytes")
+
+
+if __name__ == "__main__":
+    main()
