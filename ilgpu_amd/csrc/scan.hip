@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
 // "Differs" is Comparison<T>.Compare(a, b) != 0 (ComparisonOperations.tt:30-45),
 // i.e. CompareTo: all NaNs are equal to each other and -0.0 equals +0.0.
 #ifndef ILGPU_HIP_UNIQUE_VECS
-#define ILGPU_HIP_UNIQUE_VECS 8
+#define ILGPU_HIP_UNIQUE_VECS 12
 #endif
 constexpr int kUniqueVecs = ILGPU_HIP_UNIQUE_VECS;
 

@@ -642,6 +642,25 @@ def test_unique_random_runs(dtype):
         assert np.array_equal(kept.view(np.uint8), expect.view(np.uint8)), n
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.int32, np.int64, np.float64])
+def test_unique_tile_edges(dtype):
+    # a tile is 512 threads x 12 sixteen-byte vectors
+    tile = 512 * 12 * (16 // np.dtype(dtype).itemsize)
+    for n in sorted({tile * m + d for m in (1, 2) for d in (-1, 0, 1)}):
+        note("unique tile edge", np.dtype(dtype).name, n)
+        r = np.random.default_rng(n)
+        vals = np.repeat(r.integers(0, 100, size=n), r.integers(1, 4, size=n))[:n].astype(dtype)
+        kept, _, count = gpu_unique(vals)
+        expect = O.unique(vals)
+        assert count == expect.size, n
+        assert np.array_equal(kept.view(np.uint8), expect.view(np.uint8)), n
+    # a run that spans a whole tile and its two borders
+    vals = np.concatenate([np.arange(tile - 2), np.full(tile + 5, 7), np.arange(9)]).astype(dtype)
+    kept, _, count = gpu_unique(vals)
+    expect = O.unique(vals)
+    assert count == expect.size and np.array_equal(kept.view(np.uint8), expect.view(np.uint8))
+
+
 def test_unique_all_equal_and_all_distinct_large():
     n = (1 << 24) + 3
     kept, _, count = gpu_unique(np.full(n, 7, dtype=np.int32))
