@@ -44,7 +44,7 @@ def parse_args():
                    help="skip the other primitives")
     p.add_argument("--no-cpu", action="store_true",
                    help="skip the CPU baseline")
-    p.add_argument("--cpu-log2n", type=int, default=26,
+    p.add_argument("--cpu-log2n", type=int, default=27,
                    help="log2 of the CPU baseline sample size")
     return p.parse_args()
 
@@ -88,7 +88,7 @@ def kernel_stats(capi, name):
 # committed profile is reported for the workload it was taken on.
 MEASURED_TRAFFIC_BYTES = {
     # (kernel, log2 n): bytes per launch
-    ("onesweep_kernel<4,0>", 28): 2.395e9,
+    ("onesweep_kernel<4,0>", 28): 2.397e9,
 }
 # The same for the other workloads at their default sizes, keyed by bench name.
 MEASURED_EXTRA_TRAFFIC_BYTES = {
@@ -96,11 +96,13 @@ MEASURED_EXTRA_TRAFFIC_BYTES = {
     "reduce_add_f32_2^28": 1.074e9,
     "histogram_u8_256bins_2^30": 1.075e9,
     "histogram_i32_4096bins_2^28": 1.091e9,
-    "radix_sort_pairs_u64_u32_2^27": 3.761e9,
-    "unique_i32_all_distinct_2^28": 2.159e9,
+    "radix_sort_pairs_u64_u32_2^27": 3.680e9,
+    "unique_i32_all_distinct_2^28": 2.155e9,
     "sequence_i32_2^28": 1.074e9,
     "initialize_i32_2^28": 1.074e9,
-    "reorder_u32_random_permutation_2^28": 3.639e10,
+    "transform_negate_i32_2^28": 2.147e9,
+    "transform_i32_to_i64_2^28": 3.221e9,
+    "reorder_u32_random_permutation_2^28": 3.638e10,
 }
 
 
