@@ -188,3 +188,48 @@ def test_sort_beyond_2p30_keys():
     torch.cuda.synchronize()
     assert bool((work[:sevens] == 7).all().item())
     assert bool((work[sevens:] == 0x01000003).all().item())
+
+
+def test_maximum_length_int_max():
+    # The reference accepts views up to int.MaxValue elements
+    # (RadixSortExtensions.cs:1195-1199, ScanExtensions.cs:675-678): every
+    # primitive at exactly 2^31 - 1 elements, checked by totals and structure.
+    import torch
+    n = (1 << 31) - 1
+    dev = "cuda:0"
+    note("maximum length: 2^31 - 1 uint8 samples / keys")
+    idx = torch.arange(n, device=dev, dtype=torch.int32)
+    samples = ((idx * 37) ^ (idx >> 9)).to(torch.uint8)     # every byte value, uneven counts
+    del idx
+    # histogram: totals against chunked bincounts
+    counts = torch.zeros(256, dtype=torch.int64, device=dev)
+    for lo in range(0, n, 1 << 28):
+        counts += torch.bincount(samples[lo: lo + (1 << 28)].to(torch.int64), minlength=256)
+    bins = D.zeros(256, np.int64)
+    capi.histogram(wrap(samples, np.uint8), bins)
+    torch.cuda.synchronize()
+    assert np.array_equal(bins.numpy(), counts.cpu().numpy())
+    # sort of the same bytes: output = each value repeated count times
+    keys = samples.clone()
+    capi.radix_sort_keys(wrap(keys, np.uint8))
+    torch.cuda.synchronize()
+    starts = torch.cumsum(counts, 0) - counts
+    for v in (0, 1, 127, 128, 255):
+        s, c = int(starts[v].item()), int(counts[v].item())
+        assert bool((keys[s: s + c] == v).all().item()), v
+    assert bool((keys[1:] >= keys[:-1]).all().item())
+    del keys, samples
+    note("maximum length: 2^31 - 1 int32 scan and reduce")
+    x = (torch.arange(n, device=dev, dtype=torch.int32) & 7) - 3      # -3 .. 4
+    out = torch.empty_like(x)
+    capi.scan(wrap(x, np.int32), wrap(out, np.int32), kind=capi.SCAN_INCLUSIVE)
+    total = D.zeros(1, np.int32)
+    capi.reduce(wrap(x, np.int32), total)
+    torch.cuda.synchronize()
+    # x has period 8 with sum 4: closed form for the inclusive scan at any index
+    probe = torch.tensor([0, 1, 7, 8, 12345, (1 << 30) + 3, n - 2, n - 1], device=dev, dtype=torch.int64)
+    pre = torch.tensor([-3, -5, -6, -6, -5, -3, 0, 4], device=dev, dtype=torch.int64)
+    closed = (probe // 8) * 4 + pre[probe % 8]
+    assert bool((out[probe].to(torch.int64) == closed).all().item())
+    assert bool(((out[1:] - out[:-1]) == x[1:]).all().item())
+    assert int(total.numpy()[0]) == int(closed[-1].item())
