@@ -979,3 +979,114 @@ def test_sort_pairs_16_byte_values_tile_edges():
         order = np.argsort(keys, kind="stable")
         assert np.array_equal(dk.numpy(), keys[order]), n
         assert np.array_equal(dv.numpy(), vals[order]), n
+
+
+# ------------------------------------------------------------- streams, graphs
+def test_two_streams_run_independent_calls_concurrently():
+    # Calls on different streams with different temps must not disturb each
+    # other (the delegates are re-entrant across streams; only a temp buffer is
+    # single-use at a time).
+    import torch
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    n1, n2 = 3_000_017, 2_500_003
+    keys = random_ints(np.uint32, n1, seed=41)
+    vals = random_ints(np.int32, n2, seed=42, lo=-9, hi=9)
+    samples = random_ints(np.uint8, n2, seed=43)
+    d_keys = [D.from_numpy(keys) for _ in range(4)]
+    d_vals = D.from_numpy(vals)
+    d_scan = [D.zeros(n2, np.int32) for _ in range(4)]
+    d_bins = [D.zeros(256, np.int32) for _ in range(4)]
+    d_sum = [D.zeros(1, np.int32) for _ in range(4)]
+    d_samples = D.from_numpy(samples)
+    t_sort = capi.temp_buffer(capi.radix_sort_temp_bytes(n1, np.uint32))
+    t_scan = capi.temp_buffer(capi.scan_temp_bytes(n2, np.int32))
+    t_red = capi.temp_buffer(capi.reduce_temp_bytes(n2, np.int32))
+    torch.cuda.synchronize()
+    for i in range(4):
+        with torch.cuda.stream(s1):
+            capi.radix_sort_keys(d_keys[i], t_sort, descending=bool(i & 1))
+        with torch.cuda.stream(s2):
+            capi.scan(d_vals, d_scan[i], t_scan, kind=capi.SCAN_EXCLUSIVE)
+            capi.histogram(d_samples, d_bins[i])
+            capi.reduce(d_vals, d_sum[i], t_red)
+    s1.synchronize()
+    s2.synchronize()
+    asc = O.radix_sort(keys)
+    e_scan = O.scan(vals, inclusive=False)
+    e_bins, _ = O.histogram(samples, np.zeros(256, dtype=np.int32))
+    for i in range(4):
+        assert np.array_equal(d_keys[i].numpy(), asc[::-1] if i & 1 else asc), i
+        assert np.array_equal(d_scan[i].numpy(), e_scan), i
+        assert np.array_equal(d_bins[i].numpy(), e_bins), i
+        assert d_sum[i].numpy()[0] == O.reduce(vals), i
+
+
+def test_calls_can_be_captured_into_a_graph_and_replayed():
+    # Every call is stream-ordered kernels only (temp memory is cleared by a
+    # fill kernel, nothing is allocated), so a sequence of calls can be
+    # captured once and replayed.  Each replay runs on new input contents, with
+    # eager work and synchronisations in between, and is checked on its own.
+    import torch
+    n = 1_200_007
+    static_keys = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+    static_vals = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+    work = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+    uniq = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+    scanned = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+    bins = torch.zeros(4096, dtype=torch.int32, device="cuda:0")
+
+    def wrap(t, dt):
+        return D(t.numel(), dt, _bytes=t.view(torch.uint8))
+
+    d_work, d_uniq = wrap(work, np.uint32), wrap(uniq, np.uint32)
+    d_vals, d_scanned, d_bins = wrap(static_vals, np.int32), wrap(scanned, np.int32), wrap(bins, np.int32)
+    d_total, d_count = D.zeros(1, np.int32), D.zeros(1, np.int64)
+    t_sort = capi.temp_buffer(capi.radix_sort_temp_bytes(n, np.uint32))
+    t_scan = capi.temp_buffer(capi.scan_temp_bytes(n, np.int32))
+    t_red = capi.temp_buffer(capi.reduce_temp_bytes(n, np.int32))
+    t_uniq = capi.temp_buffer(capi.unique_temp_bytes(n, np.uint32))
+
+    def sequence_of_calls():
+        work.copy_(static_keys)
+        capi.radix_sort_keys(d_work, t_sort)
+        uniq.copy_(work)
+        capi.unique(d_uniq, d_count, t_uniq)
+        capi.scan(d_vals, d_scanned, t_scan, kind=capi.SCAN_INCLUSIVE)
+        capi.reduce(d_vals, d_total, t_red)
+        bins.zero_()
+        capi.histogram(d_vals, d_bins)
+
+    def fill(seed):
+        k = random_ints(np.uint32, n, seed=seed, lo=0, hi=50_000)
+        v = random_ints(np.int32, n, seed=seed + 1, lo=0, hi=4095)
+        static_keys.copy_(torch.from_numpy(k.view(np.int32)))
+        static_vals.copy_(torch.from_numpy(v))
+        return k, v
+
+    def check(k, v, tag):
+        torch.cuda.synchronize()
+        assert np.array_equal(d_work.numpy(), O.radix_sort(k)), tag
+        e = O.unique(O.radix_sort(k))
+        kept = int(d_count.numpy()[0])
+        assert kept == e.size and np.array_equal(d_uniq.numpy()[:kept], e), tag
+        assert np.array_equal(d_scanned.numpy(), O.scan(v)), tag
+        assert d_total.numpy()[0] == O.reduce(v), tag
+        eb, _ = O.histogram(v, np.zeros(4096, dtype=np.int32))
+        assert np.array_equal(d_bins.numpy(), eb), tag
+
+    k, v = fill(100)
+    sequence_of_calls()                      # eager, also warms the one-time queries
+    check(k, v, "eager")
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            sequence_of_calls()
+    torch.cuda.synchronize()
+    for r in range(3):
+        k, v = fill(200 + 10 * r)
+        junk = torch.rand(1 << 20, device="cuda:0").sum().item()   # eager work between replays
+        assert junk > 0
+        graph.replay()
+        check(k, v, ("replay", r))
