@@ -721,7 +721,8 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
       ++shift;
     const size_t lds = (size_t)((passes * kRadix) << shift) * 4;
     int64_t blocks = div_up(div_up(a.n, Vec16<K>::N), kHistBlock);
-    if (blocks > (int64_t)cus * 4) blocks = (int64_t)cus * 4;
+    // Two blocks of 64 KiB of counters are resident per CU: no second round.
+    if (blocks > (int64_t)cus * 2) blocks = (int64_t)cus * 2;
     if (blocks < 1) blocks = 1;
     ProfileScope scope(stream, "sort_histogram");
     hipLaunchKernelGGL((sort_histogram_kernel<K>), dim3((unsigned)blocks),
