@@ -144,10 +144,15 @@ __device__ __forceinline__ uint32_t digit_of(K k, const KeyXform& xf, int shift)
   return (uint32_t)(ordered_bits(k, xf) >> shift) & (kRadix - 1);
 }
 
+constexpr uint32_t kNoHotDigit = 0xFFFFFFFFu;
+constexpr int kMaxHot = 4;
 // Device-resident description of the passes, written by plan_kernel.
 struct SortPlan {
   uint32_t skip[kMaxPasses];        // digit identical for all keys
   uint32_t src_is_alt[kMaxPasses];  // pass reads the alternate buffer
+  // Up to kMaxHot digits that each hold an eighth of the keys or more, most
+  // frequent first; unused entries are kNoHotDigit.
+  uint32_t hot[kMaxPasses][kMaxHot];
   uint32_t first_executed;          // index of the first pass that runs
   uint32_t executed;                // number of passes that run
   uint32_t final_in_alt;            // result sits in the alternate buffer
@@ -222,15 +227,26 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
     SortPlan* __restrict__ plan, int passes, uint32_t n) {
   __shared__ uint32_t s_wave[kRadix / kWaveSize];
   __shared__ int s_trivial;
+  __shared__ unsigned long long s_hot[kMaxHot];  // count << 8 | digit, most frequent first
   const int d = threadIdx.x;
   const int lane = d & (kWaveSize - 1);
   const int wave = d / kWaveSize;
   uint32_t parity = 0, executed = 0, first = passes;
   for (int p = 0; p < passes; ++p) {
+    if (d < kMaxHot) s_hot[d] = 0ull;
     if (d == 0) s_trivial = 0;
     __syncthreads();
     const uint32_t c = global_hist[p * kRadix + d];
     if (c == n) s_trivial = 1;
+    // A digit qualifies with an eighth of the keys (two lanes of a
+    // sub-tile row on average); kMaxHot rounds of "largest below the previous
+    // one" order the most frequent ones.
+    const unsigned long long mine = ((unsigned long long)c << 8) | (unsigned long long)d;
+    const bool frequent = (uint64_t)c * 8 >= (uint64_t)n;
+    for (int h = 0; h < kMaxHot; ++h) {
+      if (frequent && (h == 0 || mine < s_hot[h - 1])) atomicMax(&s_hot[h], mine);
+      __syncthreads();
+    }
     uint32_t inc = c;
 #pragma unroll
     for (int s = 1; s < kWaveSize; s <<= 1) {
@@ -246,6 +262,8 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
     if (d == 0) {
       plan->skip[p] = trivial ? 1u : 0u;
       plan->src_is_alt[p] = parity;
+      for (int h = 0; h < kMaxHot; ++h)
+        plan->hot[p][h] = s_hot[h] != 0ull ? (uint32_t)(s_hot[h] & 0xFFull) : kNoHotDigit;
     }
     if (!trivial) {
       if (executed == 0) first = p;
@@ -312,7 +330,7 @@ __device__ __forceinline__ void load_tile_keys(
 #endif
 
 // Sorts one tile by the digit of `pass` and scatters it.
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL>
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT>
 __device__ __forceinline__ void sort_tile(
     typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
     typename KeyOf<KEY_BYTES>::type* __restrict__ dst_keys,
@@ -320,7 +338,7 @@ __device__ __forceinline__ void sort_tile(
     typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
     int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
     const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
-    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan) {
+    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan, const uint32_t (&hot)[kMaxHot]) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
@@ -384,25 +402,55 @@ __device__ __forceinline__ void sort_tile(
   // Rank inside the sub-tile, later position inside the tile: 16 bits each.
   uint32_t* my_slots = s_slot + sub * kRadix;
   uint32_t packed[kItems / 2];
+  // HOT: some digits hold a large share of the keys each (known from the
+  // global histogram).  Their keys would all meet in one slot, and LDS
+  // serialises the atomics of a wave to one address; they are ranked by one
+  // ballot per such digit instead and only the other keys go through the
+  // slots.
+  uint32_t hot_count[kMaxHot] = {};  // keys of each hot digit in this sub-tile so far
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
-    uint32_t* slot = my_slots + item_digit(j);
-    __hip_atomic_fetch_or(slot, lane_bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint32_t both = __hip_atomic_load(slot, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint32_t peers = both & kSubLaneMask;
-    const uint32_t before = both >> 16;
-    const uint32_t below = (uint32_t)__popc(peers & lower_lanes);
-    if (below == 0)  // new count, mask cleared for the next row
-      __hip_atomic_store(slot, (before + (uint32_t)__popc(peers)) << 16,
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    const uint32_t rank = before + below;
+    const uint32_t d = item_digit(j);
+    uint32_t rank = 0;
+    bool through_slot = true;
+    if constexpr (HOT) {
+#pragma unroll
+      for (int h = 0; h < kMaxHot; ++h) {
+        if (hot[h] == kNoHotDigit) continue;  // wave-uniform
+        const bool is_hot = d == hot[h];
+        const uint64_t hot_lanes = __ballot(is_hot);
+        const uint32_t mine = (uint32_t)(hot_lanes >> (lane & ~(kSubLanes - 1))) & kSubLaneMask;
+        if (is_hot) {
+          rank = hot_count[h] + (uint32_t)__popc(mine & lower_lanes);
+          through_slot = false;
+        }
+        hot_count[h] += (uint32_t)__popc(mine);
+      }
+    }
+    if (through_slot) {
+      uint32_t* slot = my_slots + d;
+      __hip_atomic_fetch_or(slot, lane_bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      const uint32_t both = __hip_atomic_load(slot, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_WORKGROUP);
+      const uint32_t peers = both & kSubLaneMask;
+      const uint32_t before = both >> 16;
+      const uint32_t below = (uint32_t)__popc(peers & lower_lanes);
+      if (below == 0)  // new count, mask cleared for the next row
+        __hip_atomic_store(slot, (before + (uint32_t)__popc(peers)) << 16,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      rank = before + below;
+    }
     if (j % 2 == 0) packed[j / 2] = rank;
     else packed[j / 2] |= rank << 16;
     // Rows chain through LDS anyway.  Pin the packed rank here: left alone,
     // the compiler sinks the rank arithmetic of all rows to where the ranks
     // are used and keeps two live registers per key until then.
     asm volatile("" : "+v"(packed[j / 2]));
+  }
+  if constexpr (HOT) {
+#pragma unroll
+    for (int h = 0; h < kMaxHot; ++h)  // these slots are untouched so far: still zero
+      if (hot[h] != kNoHotDigit && sub_lane == 0) my_slots[hot[h]] = hot_count[h] << 16;
   }
   __syncthreads();
 
@@ -566,6 +614,9 @@ void onesweep_kernel(
 
   if (plan->skip[pass]) return;
   const bool src_alt = plan->src_is_alt[pass] != 0;
+  uint32_t hot[kMaxHot];
+#pragma unroll
+  for (int h = 0; h < kMaxHot; ++h) hot[h] = plan->hot[pass][h];
   const K* src_keys = src_alt ? keys_b : keys_a;
   K* dst_keys = src_alt ? keys_a : keys_b;
   const Val* src_vals = src_alt ? vals_b : vals_a;
@@ -601,14 +652,21 @@ void onesweep_kernel(
         z[i] = make_uint4(0u, 0u, 0u, 0u);
     }
     __syncthreads();
-    if (valid == kTile) {
-      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, true>(
-          key, dst_keys, src_vals, dst_vals, tile_base, kTile, tile, pass, xf,
-          excl, status, make_index, s_stage, s_global_off, s_scan);
+    if (hot[0] == kNoHotDigit) {
+      if (valid == kTile) {
+        sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, true, false>(
+            key, dst_keys, src_vals, dst_vals, tile_base, kTile, tile, pass, xf,
+            excl, status, make_index, s_stage, s_global_off, s_scan, hot);
+      } else {
+        sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false, false>(
+            key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
+            excl, status, make_index, s_stage, s_global_off, s_scan, hot);
+      }
     } else {
-      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false>(
+      // The tail tile takes the same path: FULL only saves bounds checks.
+      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false, true>(
           key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
-          excl, status, make_index, s_stage, s_global_off, s_scan);
+          excl, status, make_index, s_stage, s_global_off, s_scan, hot);
     }
   }
 }

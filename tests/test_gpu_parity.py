@@ -981,6 +981,48 @@ def test_sort_pairs_16_byte_values_tile_edges():
         assert np.array_equal(dv.numpy(), vals[order]), n
 
 
+# ------------------------------------------------------------- dominant digits
+# A digit that holds an eighth of the keys or more is ranked by ballots instead
+# of LDS slots (up to four such digits per pass).
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.uint32, np.int64, np.float32])
+@pytest.mark.parametrize("shares", [(1.0,), (0.6, 0.4), (0.5, 0.2, 0.2), (0.25, 0.25, 0.25, 0.25),
+                                    (0.2, 0.2, 0.2, 0.2, 0.2), (0.13, 0.13)])
+def test_sort_keys_with_dominant_digits(dtype, shares):
+    r = np.random.default_rng(len(shares) * 131 + np.dtype(dtype).num)
+    for n in (1, 777, 18431, 18432, 18433, 100003, (1 << 20) + 11):
+        note("dominant digits", np.dtype(dtype).name, shares, n)
+        # chosen values differ in every byte, 0xFF bytes included (the digit of the
+        # padding keys in a partial tile); the rest of the keys are uniform
+        pool = np.array([0xFFFFFFFFFFFFFFFF, 0x0101010101010101, 0x80FF80FF80FF80FF,
+                         0x7F007F007F007F00, 0x55AA55AA55AA55AA], dtype=np.uint64)
+        which = r.choice(len(shares) + 1, size=n, p=list(shares) + [max(0.0, 1.0 - sum(shares))])
+        bits = np.where(which < len(shares), pool[np.minimum(which, len(pool) - 1)],
+                        r.integers(0, 1 << 63, size=n, dtype=np.uint64))
+        width = np.dtype(dtype).itemsize
+        keys = (bits & np.uint64((1 << (8 * width)) - 1 if width < 8 else 0xFFFFFFFFFFFFFFFF)).astype(
+            np.dtype("u%d" % width)).view(dtype)
+        for desc in (False, True):
+            d = D.from_numpy(keys)
+            capi.radix_sort_keys(d, descending=desc)
+            sync()
+            assert np.array_equal(d.numpy().view(np.uint8),
+                                  O.radix_sort(keys, descending=desc).view(np.uint8)), (n, desc)
+
+
+@pytest.mark.parametrize("kdt,vdt", [(np.uint32, np.uint32), (np.uint64, np.uint32), (np.uint16, np.uint64)])
+def test_sort_pairs_with_dominant_digits_is_stable(kdt, vdt):
+    r = np.random.default_rng(77)
+    for n in (5000, 100003, (1 << 20) + 5):
+        keys = r.choice(np.array([0, 255, 256, 0xFFFF, 12345], dtype=np.uint64), size=n,
+                        p=[0.5, 0.2, 0.15, 0.1, 0.05]).astype(kdt)
+        dk, dv = D.from_numpy(keys), D.zeros(n, vdt)
+        capi.radix_sort_pairs(dk, dv, values_from_index=True)
+        sync()
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(dk.numpy(), keys[order])
+        assert np.array_equal(dv.numpy(), order.astype(vdt))
+
+
 # ------------------------------------------------------------- streams, graphs
 def test_two_streams_run_independent_calls_concurrently():
     # Calls on different streams with different temps must not disturb each
