@@ -8,8 +8,9 @@
 // tiles per step, so tiles only wait for data, never for their turn.
 //
 // Tile layout (kBlock = 512 threads, 8 waves, kVecs = 16 16-byte vectors per
-// lane, i.e. 128 KiB per tile: time per launch falls with the number of tiles
-// until about this size, then register pressure takes over):
+// lane for 4-byte elements, i.e. 128 KiB per tile: time per launch falls with
+// the number of tiles until about this size, then register pressure takes
+// over; 10 vectors, 80 KiB, for 8-byte elements):
 //   wave w owns a contiguous chunk of kVecs*64 vectors; vector j of lane l is
 //   chunk[j*64 + l], so every load/store instruction of a wave covers 1 KiB of
 //   consecutive addresses (dwordx4 per lane).  Scan order inside a wave is
@@ -38,11 +39,21 @@ namespace {
 constexpr int kBlock = ILGPU_HIP_SCAN_BLOCK;
 constexpr int kWaves = kBlock / kWaveSize;
 constexpr int kVecs = ILGPU_HIP_SCAN_VECS;
+#ifndef ILGPU_HIP_SCAN_VECS8
+#define ILGPU_HIP_SCAN_VECS8 10
+#endif
+// 16-byte vectors per thread and tile, by element size.  8-byte elements
+// double the registers of the per-row prefixes, and their kernels run one
+// block per CU either way; 80 KiB tiles measured best for Add (2^27 int64:
+// 0.47 ms against 0.50 at 128 KiB and 0.49 at 64 KiB).
+template <typename T> constexpr int scan_vecs() {
+  return sizeof(T) == 8 ? ILGPU_HIP_SCAN_VECS8 : kVecs;
+}
 constexpr uint32_t kFlagInvalid = 0, kFlagAggregate = 1, kFlagPrefix = 2;
 constexpr int64_t kHeaderBytes = 256;  // ticket counter, padded
 
 template <typename T> constexpr int tile_elems() {
-  return kBlock * kVecs * Vec16<T>::N;
+  return kBlock * scan_vecs<T>() * Vec16<T>::N;
 }
 
 template <typename T> struct Bits;
@@ -180,6 +191,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
   using F = Functor<T, OP>;
   using V = typename Vec16<T>::type;
   constexpr int VN = Vec16<T>::N;
+  constexpr int kTileVecs = scan_vecs<T>();
   constexpr int kTile = tile_elems<T>();
   constexpr int kWaveElems = kTile / kWaves;
 
@@ -196,18 +208,18 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
   const int64_t wave_base = tile_base + (int64_t)wave * kWaveElems;
   const bool full = tile_base + kTile <= n;
 
-  T x[kVecs][VN];
+  T x[kTileVecs][VN];
   if (VECTOR && full) {
     const V* src = reinterpret_cast<const V*>(in + wave_base);
 #pragma unroll
-    for (int j = 0; j < kVecs; ++j) {
+    for (int j = 0; j < kTileVecs; ++j) {
       V v = __builtin_nontemporal_load(&src[j * kWaveSize + lane]);
 #pragma unroll
       for (int k = 0; k < VN; ++k) x[j][k] = v[k];
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < kVecs; ++j)
+    for (int j = 0; j < kTileVecs; ++j)
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
         const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
@@ -216,10 +228,10 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
   }
 
   // Lane-local inclusive scan of each vector, then one wave scan per j.
-  T lane_excl[kVecs];   // fold of the vectors of lower lanes, same j
-  T seg_total[kVecs];   // fold of the whole 64-lane row j
+  T lane_excl[kTileVecs];   // fold of the vectors of lower lanes, same j
+  T seg_total[kTileVecs];   // fold of the whole 64-lane row j
 #pragma unroll
-  for (int j = 0; j < kVecs; ++j) {
+  for (int j = 0; j < kTileVecs; ++j) {
 #pragma unroll
     for (int k = 1; k < VN; ++k) x[j][k] = F::apply(x[j][k - 1], x[j][k]);
     const T inc = wave_inclusive_scan<T, OP>(x[j][VN - 1], lane);
@@ -229,7 +241,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
   }
   T wave_total = seg_total[0];
 #pragma unroll
-  for (int j = 1; j < kVecs; ++j) wave_total = F::apply(wave_total, seg_total[j]);
+  for (int j = 1; j < kTileVecs; ++j) wave_total = F::apply(wave_total, seg_total[j]);
   if (lane == 0) s_wave_total[wave] = wave_total;
   __syncthreads();
 
@@ -250,7 +262,7 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(
   T running = F::apply(s_prefix, wave_prefix);  // prefix of row 0 of this wave
   V* dst = reinterpret_cast<V*>(out + wave_base);
 #pragma unroll
-  for (int j = 0; j < kVecs; ++j) {
+  for (int j = 0; j < kTileVecs; ++j) {
     const T before = F::apply(running, lane_excl[j]);  // prefix of x[j][0]
     T r[VN];
 #pragma unroll

@@ -981,6 +981,19 @@ def test_sort_pairs_16_byte_values_tile_edges():
         assert np.array_equal(dv.numpy(), vals[order]), n
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.int64, np.uint64])
+def test_scan_tile_edges(dtype):
+    # a tile is 512 threads x 16 sixteen-byte vectors for 4-byte elements, x 10 for 8-byte ones
+    tile = 512 * (16 * 4 if np.dtype(dtype).itemsize == 4 else 10 * 2)
+    for n in sorted({tile * m + d for m in (1, 2, 3) for d in (-1, 0, 1)}):
+        vals = random_ints(dtype, n, seed=n)
+        for op in (capi.OP_ADD, capi.OP_MAX, capi.OP_MIN):
+            for inclusive in (True, False):
+                note("scan tile edge", np.dtype(dtype).name, n, op, inclusive)
+                got = gpu_scan(vals, op, inclusive)
+                assert np.array_equal(got[:n], O.scan(vals, op=op, inclusive=inclusive)), (n, op, inclusive)
+
+
 # ------------------------------------------------------------- dominant digits
 # A digit that holds an eighth of the keys or more is ranked by ballots instead
 # of LDS slots (up to four such digits per pass).
