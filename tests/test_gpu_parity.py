@@ -1036,6 +1036,40 @@ def test_sort_pairs_with_dominant_digits_is_stable(kdt, vdt):
         assert np.array_equal(dv.numpy(), order.astype(vdt))
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.uint16, np.uint32, np.int64, np.float64])
+@pytest.mark.parametrize("run", [2, 15, 16, 17, 64, 1000])
+def test_sort_keys_in_runs_and_presorted(dtype, run):
+    # Rows of sixteen neighbouring keys that share a digit take a shortcut in the
+    # ranking: runs around the row length, runs that straddle rows, sorted and
+    # reversed inputs.
+    r = np.random.default_rng(run)
+    for n in (run, 18432 + run // 2, 100003, (1 << 20) + 7):
+        note("runs", np.dtype(dtype).name, run, n)
+        starts = r.integers(0, 1 << 62, size=n // run + 2, dtype=np.uint64)
+        bits = np.repeat(starts, run)[r.integers(0, run):][:n]
+        width = np.dtype(dtype).itemsize
+        keys = (bits >> np.uint64(64 - 8 * width)).astype(np.dtype("u%d" % width)).view(dtype)
+        if np.dtype(dtype).kind == "f":
+            keys = np.where(np.isnan(keys), np.dtype(dtype).type(1.5), keys)
+        for variant in (keys, np.sort(keys), np.sort(keys)[::-1].copy()):
+            d = D.from_numpy(variant)
+            capi.radix_sort_keys(d)
+            sync()
+            assert np.array_equal(d.numpy().view(np.uint8), O.radix_sort(variant).view(np.uint8)), n
+
+
+def test_sort_pairs_in_runs_is_stable():
+    r = np.random.default_rng(5)
+    for n in (40000, (1 << 20) + 3):
+        keys = np.repeat(r.integers(0, 1 << 20, size=n // 50 + 1), 50)[:n].astype(np.uint32)
+        dk, dv = D.from_numpy(keys), D.zeros(n, np.uint32)
+        capi.radix_sort_pairs(dk, dv, values_from_index=True)
+        sync()
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(dk.numpy(), keys[order])
+        assert np.array_equal(dv.numpy(), order.astype(np.uint32))
+
+
 # ------------------------------------------------------------- streams, graphs
 def test_two_streams_run_independent_calls_concurrently():
     # Calls on different streams with different temps must not disturb each
