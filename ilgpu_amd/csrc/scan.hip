@@ -22,8 +22,9 @@
 // eight XCDs of the device have separate L2s.
 //   4-byte T: one 64-bit word {flag, value} per tile;
 //   8-byte T: two such words per tile, one per half of the value.
+// Each tile's words sit in a 128-byte line of their own.
 //
-// Algorithmic HBM traffic: 2 * n * sizeof(T) bytes (status words: 8 B/tile).
+// Algorithmic HBM traffic: 2 * n * sizeof(T) bytes (status: 128 B/tile).
 #include "kernels.hpp"
 
 namespace ilgpu_hip {
@@ -36,6 +37,13 @@ namespace {
 #ifndef ILGPU_HIP_SCAN_VECS
 #define ILGPU_HIP_SCAN_VECS 16
 #endif
+// 8-byte status words per tile: one 128-byte line each.  Every resident block
+// polls the words of the few dozen tiles before it with loads that go past the
+// L2; packed eight bytes apart those words share a handful of lines, and the
+// memory channels that hold them fall behind on the data streams (measured at
+// 2^28 int32: 0.384 ms packed, 0.363 at 64 bytes per tile, 0.360 at 128 to 512).
+constexpr int kStatusStride = 16;
+constexpr int64_t kStatusBytes = 8 * kStatusStride;
 constexpr int kBlock = ILGPU_HIP_SCAN_BLOCK;
 constexpr int kWaves = kBlock / kWaveSize;
 constexpr int kVecs = ILGPU_HIP_SCAN_VECS;
@@ -84,14 +92,14 @@ template <typename T> struct TileState<T, 4> {
   uint64_t* words;
   __device__ __forceinline__ void publish(int tile, uint32_t flag, T v) const {
     const uint64_t w = ((uint64_t)flag << 32) | to_bits(v);
-    __hip_atomic_store(&words[tile], w, __ATOMIC_RELAXED,
+    __hip_atomic_store(&words[(int64_t)tile * kStatusStride], w, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
   }
   // Spins until the tile has published something; returns its flag.
   __device__ __forceinline__ uint32_t wait(int tile, T* v) const {
     uint64_t w;
     while (true) {
-      w = __hip_atomic_load(&words[tile], __ATOMIC_RELAXED,
+      w = __hip_atomic_load(&words[(int64_t)tile * kStatusStride], __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_AGENT);
       if ((uint32_t)(w >> 32) != kFlagInvalid) break;
       __builtin_amdgcn_s_sleep(1);
@@ -101,27 +109,28 @@ template <typename T> struct TileState<T, 4> {
   }
 };
 
-// 8-byte values: two 64-bit words per tile, {flag, low half} and {flag, high
-// half}, each written and read with one relaxed atomic.  A tile writes each
+// 8-byte values: two 64-bit words in the tile's line, {flag, low half} and
+// {flag, high half}, each written and read with one relaxed atomic.  A tile writes each
 // state (aggregate, then prefix) once, so two words with the same flag hold
 // the halves of the same value; a reader that catches the words in different
 // states reads again.  No fences: an agent-scope release would write back the
 // whole L2 of the XCD for every tile.
 template <typename T> struct TileState<T, 8> {
-  uint64_t* low;
-  uint64_t* high;
+  uint64_t* words;
   __device__ __forceinline__ void publish(int tile, uint32_t flag, T v) const {
     const uint64_t bits = to_bits(v);
-    __hip_atomic_store(&low[tile], ((uint64_t)flag << 32) | (uint32_t)bits,
+    uint64_t* w = &words[(int64_t)tile * kStatusStride];
+    __hip_atomic_store(&w[0], ((uint64_t)flag << 32) | (uint32_t)bits,
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&high[tile], ((uint64_t)flag << 32) | (bits >> 32),
+    __hip_atomic_store(&w[1], ((uint64_t)flag << 32) | (bits >> 32),
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __device__ __forceinline__ uint32_t wait(int tile, T* v) const {
     uint64_t lo, hi;
+    const uint64_t* w = &words[(int64_t)tile * kStatusStride];
     while (true) {
-      lo = __hip_atomic_load(&low[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      hi = __hip_atomic_load(&high[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      lo = __hip_atomic_load(&w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      hi = __hip_atomic_load(&w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if ((uint32_t)(lo >> 32) != kFlagInvalid && (lo >> 32) == (hi >> 32)) break;
       __builtin_amdgcn_s_sleep(1);
     }
@@ -130,15 +139,48 @@ template <typename T> struct TileState<T, 8> {
   }
 };
 
-template <typename T, int OP>
-__device__ __forceinline__ T wave_inclusive_scan(T v, int lane) {
-  using F = Functor<T, OP>;
-#pragma unroll
-  for (int d = 1; d < kWaveSize; d <<= 1) {
-    T o = shfl_up(v, d);
-    if (lane >= d) v = F::apply(o, v);
+// Data-parallel-primitive move: lane i receives `v` of the lane that the
+// control word CTRL names (row_shr:n = 0x110 + n within rows of 16 lanes,
+// row_bcast:15 = 0x142, row_bcast:31 = 0x143, wave_shr:1 = 0x138); lanes
+// without a source, and rows outside ROW_MASK, receive `fill`.
+template <typename T, int CTRL, int ROW_MASK>
+__device__ __forceinline__ T dpp_move(T fill, T v) {
+  if constexpr (sizeof(T) == 8) {
+    union { T t; int32_t w[2]; } f, a, b;
+    f.t = fill;
+    a.t = v;
+    b.w[0] = __builtin_amdgcn_update_dpp(f.w[0], a.w[0], CTRL, ROW_MASK, 0xf, false);
+    b.w[1] = __builtin_amdgcn_update_dpp(f.w[1], a.w[1], CTRL, ROW_MASK, 0xf, false);
+    return b.t;
+  } else {
+    union { T t; int32_t w; } f, a, b;
+    f.t = fill;
+    a.t = v;
+    b.w = __builtin_amdgcn_update_dpp(f.w, a.w, CTRL, ROW_MASK, 0xf, false);
+    return b.t;
   }
+}
+
+// Inclusive scan over the 64 lanes of a wave: four shifted steps inside each
+// row of 16 lanes, then the last lane of row 0 (2) is folded into row 1 (3),
+// then lane 31 into rows 2 and 3.
+template <typename T, int OP>
+__device__ __forceinline__ T wave_inclusive_scan(T v, int) {
+  using F = Functor<T, OP>;
+  const T id = F::identity();
+  v = F::apply(dpp_move<T, 0x111, 0xf>(id, v), v);
+  v = F::apply(dpp_move<T, 0x112, 0xf>(id, v), v);
+  v = F::apply(dpp_move<T, 0x114, 0xf>(id, v), v);
+  v = F::apply(dpp_move<T, 0x118, 0xf>(id, v), v);
+  v = F::apply(dpp_move<T, 0x142, 0xa>(id, v), v);
+  v = F::apply(dpp_move<T, 0x143, 0xc>(id, v), v);
   return v;
+}
+
+// Value of the previous lane; lane 0 receives `fill`.
+template <typename T>
+__device__ __forceinline__ T lane_shift_up(T fill, T v) {
+  return dpp_move<T, 0x138, 0xf>(fill, v);
 }
 
 template <typename T, int OP>
@@ -206,10 +248,16 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
   __syncthreads();
   const int tile = s_tile;
   const int lane = threadIdx.x & (kWaveSize - 1);
-  const int wave = threadIdx.x / kWaveSize;
+  // The wave index and everything derived from it are wave-uniform: kept in
+  // scalar registers, so a lane addresses its vectors by one 32-bit offset.
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
   const int64_t tile_base = (int64_t)tile * kTile;
   const int64_t wave_base = tile_base + (int64_t)wave * kWaveElems;
   const bool full = tile_base + kTile <= n;
+  // Elements of this wave's chunk that lie inside the view (tail path only).
+  const int wave_valid =
+      (int)(n - wave_base < kWaveElems ? (n - wave_base < 0 ? 0 : n - wave_base)
+                                       : kWaveElems);
 
   T x[kTileVecs][VN];
   if (VECTOR && full) {
@@ -225,8 +273,8 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
     for (int j = 0; j < kTileVecs; ++j)
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
-        const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
-        x[j][k] = idx < n ? in[idx * in_stride] : F::identity();
+        const int e = (j * kWaveSize + lane) * VN + k;
+        x[j][k] = e < wave_valid ? in[(wave_base + e) * in_stride] : F::identity();
       }
   }
 
@@ -239,8 +287,7 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
     for (int k = 1; k < VN; ++k) x[j][k] = F::apply(x[j][k - 1], x[j][k]);
     const T inc = wave_inclusive_scan<T, OP>(x[j][VN - 1], lane);
     seg_total[j] = shfl(inc, kWaveSize - 1);
-    const T up = shfl_up(inc, 1);
-    lane_excl[j] = lane == 0 ? F::identity() : up;
+    lane_excl[j] = lane_shift_up<T>(F::identity(), inc);
   }
   T wave_total = seg_total[0];
 #pragma unroll
@@ -281,8 +328,8 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
     } else {
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
-        const int64_t idx = wave_base + (int64_t)(j * kWaveSize + lane) * VN + k;
-        if (idx < n) out[idx * out_stride] = r[k];
+        const int e = (j * kWaveSize + lane) * VN + k;
+        if (e < wave_valid) out[(wave_base + e) * out_stride] = r[k];
       }
     }
     running = F::apply(running, seg_total[j]);
@@ -448,15 +495,8 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t in_stride,
   char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)temp, 256));
   uint32_t* ticket = reinterpret_cast<uint32_t*>(base);
   TileState<T> st;
-  int64_t zero_words;
-  if constexpr (sizeof(T) == 4) {
-    st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
-    zero_words = (kHeaderBytes + tiles * 8) / 4;
-  } else {
-    st.low = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
-    st.high = st.low + tiles;
-    zero_words = (kHeaderBytes + tiles * 16) / 4;
-  }
+  st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
+  const int64_t zero_words = (kHeaderBytes + tiles * kStatusBytes) / 4;
   int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
                                  zero_words);
   if (rc != ILGPU_HIP_SUCCESS) return rc;
@@ -515,12 +555,9 @@ int32_t launch_zero_words(hipStream_t stream, uint32_t* words, int64_t count) {
 
 int64_t scan_temp_bytes(int64_t n, int elem_bytes) {
   // 256 bytes of alignment slack + header + per-tile state.
-  if (elem_bytes == 4) {
-    const int64_t tiles = num_tiles<uint32_t>(n);
-    return 256 + kHeaderBytes + tiles * 8;
-  }
-  const int64_t tiles = num_tiles<uint64_t>(n);
-  return 256 + kHeaderBytes + tiles * 16;
+  const int64_t tiles =
+      elem_bytes == 4 ? num_tiles<uint32_t>(n) : num_tiles<uint64_t>(n);
+  return 256 + kHeaderBytes + tiles * kStatusBytes;
 }
 
 int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
@@ -539,7 +576,7 @@ int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
 
 int64_t unique_temp_bytes(int64_t n, int elem_bytes) {
   const int64_t tile = (int64_t)kBlock * kUniqueVecs * (16 / elem_bytes);
-  return 256 + kHeaderBytes + div_up(n, tile) * 8;
+  return 256 + kHeaderBytes + div_up(n, tile) * kStatusBytes;
 }
 
 namespace {
@@ -552,7 +589,7 @@ int32_t launch_unique_typed(hipStream_t stream, void* data, int64_t n,
   TileState<uint32_t> st;
   st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
   const int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
-                                       (kHeaderBytes + tiles * 8) / 4);
+                                       (kHeaderBytes + tiles * kStatusBytes) / 4);
   if (rc != ILGPU_HIP_SUCCESS) return rc;
   const bool vector = (reinterpret_cast<uintptr_t>(data) & 15) == 0;
   ProfileScope scope(stream, "unique");
