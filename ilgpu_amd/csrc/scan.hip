@@ -356,7 +356,19 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
 #ifndef ILGPU_HIP_UNIQUE_VECS
 #define ILGPU_HIP_UNIQUE_VECS 12
 #endif
-constexpr int kUniqueVecs = ILGPU_HIP_UNIQUE_VECS;
+#ifndef ILGPU_HIP_UNIQUE_VECS1
+#define ILGPU_HIP_UNIQUE_VECS1 4
+#endif
+#ifndef ILGPU_HIP_UNIQUE_VECS2
+#define ILGPU_HIP_UNIQUE_VECS2 8
+#endif
+// 16-byte vectors per thread and tile, by element size: every element of a
+// vector is unpacked into a register of its own, so a vector of bytes costs
+// sixteen registers and one of 2-byte elements eight.
+constexpr int unique_vecs(int elem_bytes) {
+  return elem_bytes == 1 ? ILGPU_HIP_UNIQUE_VECS1
+                         : elem_bytes == 2 ? ILGPU_HIP_UNIQUE_VECS2 : ILGPU_HIP_UNIQUE_VECS;
+}
 
 template <typename T> struct is_float_like { static constexpr bool value = is_fp<T>::value; };
 template <> struct is_float_like<_Float16> { static constexpr bool value = true; };
@@ -367,7 +379,7 @@ template <typename T> __device__ __forceinline__ bool differs(T a, T b) {
 }
 
 template <typename T> constexpr int unique_tile_elems() {
-  return kBlock * kUniqueVecs * Vec16<T>::N;
+  return kBlock * unique_vecs(sizeof(T)) * Vec16<T>::N;
 }
 
 template <typename T, bool VECTOR>
@@ -376,6 +388,7 @@ __global__ __launch_bounds__(kBlock) void unique_kernel(
     uint32_t* __restrict__ ticket, TileState<uint32_t> st, int num_tiles) {
   using V = typename Vec16<T>::type;
   constexpr int VN = Vec16<T>::N;
+  constexpr int kUniqueVecs = unique_vecs(sizeof(T));
   constexpr int kTile = unique_tile_elems<T>();
   constexpr int kWaveElems = kTile / kWaves;
 
@@ -575,7 +588,7 @@ int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
 }
 
 int64_t unique_temp_bytes(int64_t n, int elem_bytes) {
-  const int64_t tile = (int64_t)kBlock * kUniqueVecs * (16 / elem_bytes);
+  const int64_t tile = (int64_t)kBlock * unique_vecs(elem_bytes) * (16 / elem_bytes);
   return 256 + kHeaderBytes + div_up(n, tile) * kStatusBytes;
 }
 

@@ -644,8 +644,9 @@ def test_unique_random_runs(dtype):
 
 @pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.int32, np.int64, np.float64])
 def test_unique_tile_edges(dtype):
-    # a tile is 512 threads x 12 sixteen-byte vectors
-    tile = 512 * 12 * (16 // np.dtype(dtype).itemsize)
+    # a tile is 512 threads x 12 sixteen-byte vectors (4 for 1-byte elements, 8 for 2-byte ones)
+    size = np.dtype(dtype).itemsize
+    tile = 512 * {1: 4, 2: 8}.get(size, 12) * (16 // size)
     for n in sorted({tile * m + d for m in (1, 2) for d in (-1, 0, 1)}):
         note("unique tile edge", np.dtype(dtype).name, n)
         r = np.random.default_rng(n)
