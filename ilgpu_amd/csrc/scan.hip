@@ -8,9 +8,8 @@
 // tiles per step, so tiles only wait for data, never for their turn.
 //
 // Tile layout (kBlock = 512 threads, 8 waves, kVecs = 16 16-byte vectors per
-// lane for 4-byte elements, i.e. 128 KiB per tile: time per launch falls with
-// the number of tiles until about this size, then register pressure takes
-// over; 10 vectors, 80 KiB, for 8-byte elements):
+// lane, i.e. 128 KiB per tile: time per launch falls with the number of tiles
+// until about this size, then register pressure takes over):
 //   wave w owns a contiguous chunk of kVecs*64 vectors; vector j of lane l is
 //   chunk[j*64 + l], so every load/store instruction of a wave covers 1 KiB of
 //   consecutive addresses (dwordx4 per lane).  Scan order inside a wave is
@@ -48,12 +47,12 @@ constexpr int kBlock = ILGPU_HIP_SCAN_BLOCK;
 constexpr int kWaves = kBlock / kWaveSize;
 constexpr int kVecs = ILGPU_HIP_SCAN_VECS;
 #ifndef ILGPU_HIP_SCAN_VECS8
-#define ILGPU_HIP_SCAN_VECS8 10
+#define ILGPU_HIP_SCAN_VECS8 16
 #endif
-// 16-byte vectors per thread and tile, by element size.  8-byte elements
-// double the registers of the per-row prefixes, and their kernels run one
-// block per CU either way; 80 KiB tiles measured best for Add (2^27 int64:
-// 0.47 ms against 0.50 at 128 KiB and 0.49 at 64 KiB).
+// 16-byte vectors per thread and tile, by element size (the same 128 KiB tile
+// for both: measured at 2^27 int64 in the register-lean form, 10 vectors
+// 0.456 ms, 12: 0.401, 14: 0.394, 16: 0.382, 18 and 20 the same as 16 for Add
+// but 0.48 and 0.54 for the floating-point Max, which then spills).
 template <typename T> constexpr int scan_vecs() {
   return sizeof(T) == 8 ? ILGPU_HIP_SCAN_VECS8 : kVecs;
 }
@@ -177,6 +176,39 @@ __device__ __forceinline__ T wave_inclusive_scan(T v, int) {
   return v;
 }
 
+// Value of `v` in lane `src` as a wave-uniform (scalar register) value.
+template <typename T>
+__device__ __forceinline__ T read_lane(T v, int src) {
+  if constexpr (sizeof(T) == 8) {
+    union { T t; int32_t w[2]; } a, b;
+    a.t = v;
+    b.w[0] = __builtin_amdgcn_readlane(a.w[0], src);
+    b.w[1] = __builtin_amdgcn_readlane(a.w[1], src);
+    return b.t;
+  } else {
+    union { T t; int32_t w; } a, b;
+    a.t = v;
+    b.w = __builtin_amdgcn_readlane(a.w, src);
+    return b.t;
+  }
+}
+
+// Keeps a value where it is in program order: the scheduler otherwise
+// interleaves the row scans of a tile and keeps a copy of every row alive.
+template <typename T> __device__ __forceinline__ void pin(T& v) {
+  if constexpr (sizeof(T) == 8) {
+    union { T t; int32_t w[2]; } a;
+    a.t = v;
+    asm volatile("" : "+v"(a.w[0]), "+v"(a.w[1]));
+    v = a.t;
+  } else {
+    union { T t; int32_t w; } a;
+    a.t = v;
+    asm volatile("" : "+v"(a.w));
+    v = a.t;
+  }
+}
+
 // Value of the previous lane; lane 0 receives `fill`.
 template <typename T>
 __device__ __forceinline__ T lane_shift_up(T fill, T v) {
@@ -278,6 +310,73 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
       }
   }
 
+  if constexpr (sizeof(T) == 8) {
+    // Register-lean form for 8-byte elements, whose per-row prefixes would
+    // take two registers each: the prefix of the lower lanes is folded into
+    // the row at once, so no per-row prefix outlives this loop, and the row
+    // totals are wave-uniform values in scalar registers (104 registers at 16
+    // vectors; 2^27 int64 Add 0.419 -> 0.382 ms against the form below at 10
+    // vectors).  For 4-byte elements the two forms measure the same.
+    T seg_total[kTileVecs];
+#pragma unroll
+    for (int j = 0; j < kTileVecs; ++j) {
+#pragma unroll
+      for (int k = 1; k < VN; ++k) x[j][k] = F::apply(x[j][k - 1], x[j][k]);
+      const T inc = wave_inclusive_scan<T, OP>(x[j][VN - 1], lane);
+      seg_total[j] = read_lane<T>(inc, kWaveSize - 1);
+      const T up = lane_shift_up<T>(F::identity(), inc);
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        x[j][k] = F::apply(up, x[j][k]);
+        pin(x[j][k]);
+      }
+    }
+    T wave_total = seg_total[0];
+#pragma unroll
+    for (int j = 1; j < kTileVecs; ++j) wave_total = F::apply(wave_total, seg_total[j]);
+    if (lane == 0) s_wave_total[wave] = wave_total;
+    __syncthreads();
+    T wave_prefix = F::identity();
+    T block_total = s_wave_total[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      if (w == wave) wave_prefix = block_total;
+      block_total = F::apply(block_total, s_wave_total[w]);
+    }
+    if (wave == 0) {
+      const T exclusive = resolve_prefix<T, OP>(st, tile, block_total, lane);
+      if (lane == 0) s_prefix = exclusive;
+    }
+    __syncthreads();
+    T running = F::apply(s_prefix, wave_prefix);
+    V* dst = reinterpret_cast<V*>(out + wave_base);
+#pragma unroll
+    for (int j = 0; j < kTileVecs; ++j) {
+      T r[VN];
+      if (inclusive) {
+#pragma unroll
+        for (int k = 0; k < VN; ++k) r[k] = F::apply(running, x[j][k]);
+      } else {
+        r[0] = F::apply(running, lane_shift_up<T>(F::identity(), x[j][VN - 1]));
+#pragma unroll
+        for (int k = 1; k < VN; ++k) r[k] = F::apply(running, x[j][k - 1]);
+      }
+      if (VECTOR && full) {
+        V v;
+#pragma unroll
+        for (int k = 0; k < VN; ++k) v[k] = r[k];
+        __builtin_nontemporal_store(v, &dst[j * kWaveSize + lane]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          const int e = (j * kWaveSize + lane) * VN + k;
+          if (e < wave_valid) out[(wave_base + e) * out_stride] = r[k];
+        }
+      }
+      running = F::apply(running, seg_total[j]);
+    }
+    return;
+  }
   // Lane-local inclusive scan of each vector, then one wave scan per j.
   T lane_excl[kTileVecs];   // fold of the vectors of lower lanes, same j
   T seg_total[kTileVecs];   // fold of the whole 64-lane row j
