@@ -44,6 +44,7 @@ EXPORTS = [
     "ilgpu_hip_profile_query", "ilgpu_hip_radix_sort_temp_bytes",
     "ilgpu_hip_radix_sort_temp_bytes_strided",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
+    "ilgpu_hip_selftest_lds_atomic_order",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
     "ilgpu_hip_unique_temp_bytes", "ilgpu_hip_unique", "ilgpu_hip_initialize",
@@ -128,6 +129,8 @@ def lib() -> ctypes.CDLL:
         L.ilgpu_hip_radix_sort_keys.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64]
         L.ilgpu_hip_radix_sort_pairs.argtypes = [
             vp, vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, i64]
+        L.ilgpu_hip_selftest_lds_atomic_order.argtypes = [vp, i32, vp]
+        L.ilgpu_hip_selftest_lds_atomic_order.restype = i32
         L.ilgpu_hip_scan_temp_bytes.argtypes = [i64, i32, p64]
         L.ilgpu_hip_scan.argtypes = [vp, vp, i64, i64, vp, i64, i64, i32, i32,
                                      i32, vp, i64]
@@ -299,6 +302,13 @@ def radix_sort_pairs(keys: DeviceArray, values: DeviceArray,
         keys.type_code, values.dtype.itemsize, flags,
         VALUES_FROM_INDEX if values_from_index else VALUES_FROM_VIEW,
         temp.ptr, temp.nbytes))
+
+
+def selftest_lds_atomic_order(rows: int = 256, *, stream=None) -> int:
+    """Lanes of the LDS atomics found out of lane order (0 on gfx950)."""
+    out = DeviceArray.zeros(1, np.int64)
+    check(lib().ilgpu_hip_selftest_lds_atomic_order(_stream_ptr(stream), rows, out.ptr))
+    return int(out.numpy()[0])
 
 
 def scan_temp_bytes(n: int, dtype) -> int:

@@ -262,6 +262,15 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void* keys,
   return launch_radix_sort(static_cast<hipStream_t>(stream), a);
 }
 
+int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
+                                            int32_t rows, int64_t* mismatches) {
+  if (mismatches == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (rows < 1 || rows > (1 << 20)) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(mismatches, 8)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  return launch_lds_atomic_order_selftest(static_cast<hipStream_t>(stream), rows,
+                                          mismatches);
+}
+
 /* ---- scan -------------------------------------------------------------- */
 
 int32_t ilgpu_hip_scan_temp_bytes(int64_t n, int32_t elem_type,

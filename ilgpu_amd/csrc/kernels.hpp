@@ -44,6 +44,10 @@ int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
                               int64_t key_stride = 1, int64_t value_stride = 1);
 int64_t radix_sort_max_length();
 int32_t launch_radix_sort(hipStream_t stream, const SortArgs& args);
+// Device check of the LDS behaviour the sort's ranking relies on: lanes of one
+// returning LDS atomic that share an address are served in lane order.
+// mismatches[0] (device) receives the number of lanes found out of order.
+int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches);
 
 // scan.hip: Unique (consecutive duplicates removed in place, new length to
 // out_length[0] on the device).

@@ -13,8 +13,9 @@
 //   plan      one block turns the histograms into exclusive digit offsets,
 //             marks passes whose digit is the same for every key (they are
 //             skipped) and records which buffer each pass reads;
-//   pass x k  onesweep: a block takes a tile by ticket, ranks its keys
-//             (per-quarter-wave {count, peer mask} slots in LDS, so equal digits
+//   pass x k  onesweep: a block takes a tile by ticket, ranks its keys (one
+//             returning LDS add per key on per-wave digit counters; the LDS
+//             serves the lanes of an instruction in lane order, so equal digits
 //             keep memory order: every pass is stable), publishes
 //             its 256 digit counts, resolves the counts of all earlier tiles by
 //             decoupled look-back, stages the tile in digit order through LDS
@@ -32,6 +33,7 @@
 // Algorithmic HBM traffic for n keys of k bytes, values of v bytes and P
 // executed passes: n * (k * (2P + 1) + v * 2P) bytes.
 #include <atomic>
+#include <type_traits>
 
 #include "kernels.hpp"
 
@@ -42,7 +44,7 @@ namespace {
 constexpr int kRadix = 256;
 constexpr int kMaxPasses = 8;
 // Launch shape of the onesweep pass.  The block size fixes the number of
-// quarter-wave sub-tiles (and with it the LDS footprint of the ranking slots);
+// per-wave sub-tiles (and with it the LDS footprint of the ranking counters);
 // items per thread fix the tile size.
 #ifndef ILGPU_HIP_SORT_BLOCK
 #define ILGPU_HIP_SORT_BLOCK 512
@@ -56,11 +58,23 @@ constexpr int kMaxPasses = 8;
 #ifndef ILGPU_HIP_SORT_LOOKBACK
 #define ILGPU_HIP_SORT_LOOKBACK 4
 #endif
+// Rows whose LDS operations are in flight together while ranking, and staged
+// keys a thread reads per batch of the write-out.
+#ifndef ILGPU_HIP_SORT_RANK_GROUP
+#define ILGPU_HIP_SORT_RANK_GROUP 6
+#endif
+#ifndef ILGPU_HIP_SORT_PAIR_RANK_GROUP
+#define ILGPU_HIP_SORT_PAIR_RANK_GROUP 2
+#endif
+#ifndef ILGPU_HIP_SORT_PAIR_WRITE_GROUP
+#define ILGPU_HIP_SORT_PAIR_WRITE_GROUP 4
+#endif
+#ifndef ILGPU_HIP_SORT_WRITE_GROUP
+#define ILGPU_HIP_SORT_WRITE_GROUP 12
+#endif
 constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;
-// Lanes that rank together (a sub-tile row): a quarter of a wave, so that a
-// peer mask and a running count share one 32-bit LDS word.
-constexpr int kSubLanes = 16;
-constexpr uint32_t kSubLaneMask = (1u << kSubLanes) - 1u;
+// Lanes that rank together (a sub-tile row): one wave.
+constexpr int kSubLanes = kWaveSize;
 constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
 constexpr int kHistBlock = 512;
 #ifndef ILGPU_HIP_SORT_HIST_LDS_WORDS
@@ -280,33 +294,31 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 }
 
 // ---- onesweep pass ---------------------------------------------------------
-// Ranking.  A block's tile is cut into sub-tiles, one per quarter-wave (16
-// lanes); lane l of quarter-wave q holds items q*16*kItems + j*16 + l, j = 0
-// .. kItems-1, so memory order inside a sub-tile is (row j, lane).  Every
-// (quarter-wave, digit) pair owns one 32-bit LDS slot: a 16-bit peer mask
-// under a 16-bit running count.  For row j every lane
-//   1. ORs its lane bit into the slot of its digit (LDS atomic),
-//   2. reads the slot back: the mask now names all lanes of the quarter-wave
-//      holding that digit in this row, the count is the number of keys with
-//      the digit in earlier rows,
-//   3. ranks itself: count + number of peers in lower lanes,
-//   4. and the lowest peer stores count + number of peers with the mask
-//      cleared for the next row.
-// LDS instructions of one wave execute in issue order, so the rows chain
-// through the slot without barriers, and equal digits keep memory order: the
-// pass is stable.  No ballots: the cost per key is three LDS operations on
-// 32-bit words (the cheapest the LDS offers for scattered addresses) and
-// about ten VALU operations whatever the key distribution.
+// Ranking.  A block's tile is cut into sub-tiles, one per wave; lane l of wave
+// w holds items w*64*kItems + j*64 + l, j = 0 .. kItems-1, so memory order
+// inside a sub-tile is (row j, lane) and a row is one 256-byte load.  Every
+// (wave, digit) pair owns one 32-bit LDS counter.  For row j every lane adds
+// one to the counter of its digit with a returning LDS atomic; the value that
+// comes back is the key's rank among the keys of that digit in the sub-tile.
+//
+// That the rank follows memory order rests on two properties of the LDS:
+// instructions of one wave execute in issue order (rows chain through the
+// counters without barriers), and the lanes of ONE atomic instruction that
+// meet in one address are served in ascending lane order.  The second is a
+// property of this hardware (gfx950), not of the programming model; it is
+// checked on the device by ilgpu_hip_selftest_lds_atomic_order and, end to
+// end, by every stability test of the pair sorts.  With it the pass is stable
+// at one LDS operation per key and no cross-lane arithmetic.
 template <int KEY_BYTES, int VALUE_BYTES> struct SortTile {
   static constexpr int kSubTiles = kSortBlock / kSubLanes;
-  static constexpr int kSlotWords = kSubTiles * kRadix;
-  static constexpr int kSlotBytes = kSlotWords * 4;
+  static constexpr int kCounterWords = kSubTiles * kRadix;
+  static constexpr int kCounterBytes = kCounterWords * 4;
   static constexpr int kItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
   static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES);
   static constexpr int kSubTileKeys = kSubLanes * kItems;
   static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
   static constexpr int kStageBytes =
-      kSlotBytes > kKeyStageBytes ? kSlotBytes : kKeyStageBytes;
+      kCounterBytes > kKeyStageBytes ? kCounterBytes : kKeyStageBytes;
 };
 
 template <int KEY_BYTES, int ITEMS, bool FULL>
@@ -353,8 +365,8 @@ __device__ __forceinline__ void sort_tile(
                 "ranks and tile positions are packed two to a register");
   static_assert(kItems * kSubLanes < 65536, "a sub-tile's digit count fits 16 bits");
 
-  // Slot of (sub-tile, digit): running count << 16 | peer mask.
-  uint32_t* s_slot = reinterpret_cast<uint32_t*>(s_stage);
+  // Counter of (sub-tile, digit): keys of that digit in the rows ranked so far.
+  uint32_t* s_counter = reinterpret_cast<uint32_t*>(s_stage);
   K* s_keys = reinterpret_cast<K*>(s_stage);
   Val* s_vals = reinterpret_cast<Val*>(s_stage);
 
@@ -365,11 +377,8 @@ __device__ __forceinline__ void sort_tile(
   asm volatile("" : "+v"(tid));
   const int lane = tid & (kWaveSize - 1);
   const int wave = tid / kWaveSize;
-  const int sub = tid / kSubLanes;          // quarter-wave index in the block
-  const int sub_lane = tid % kSubLanes;
-  const uint32_t lane_bit = 1u << sub_lane;
-  const uint32_t lower_lanes = lane_bit - 1u;
-  const int first_local = sub * TileCfg::kSubTileKeys + sub_lane;
+  const int sub = wave;                     // sub-tile index in the block
+  const int first_local = sub * TileCfg::kSubTileKeys + lane;
   const int shift = pass * 8;
 
   auto digit = [&](K k) -> uint32_t {
@@ -400,81 +409,88 @@ __device__ __forceinline__ void sort_tile(
   }
 
   // Rank inside the sub-tile, later position inside the tile: 16 bits each.
-  uint32_t* my_slots = s_slot + sub * kRadix;
+  uint32_t* my_counters = s_counter + sub * kRadix;
   uint32_t packed[kItems / 2];
   // HOT: some digits hold a large share of the keys each (known from the
-  // global histogram).  Their keys would all meet in one slot, and LDS
+  // global histogram).  Their keys would all meet in one counter, and LDS
   // serialises the atomics of a wave to one address; they are ranked by one
   // ballot per such digit instead and only the other keys go through the
-  // slots.
+  // counters.
   uint32_t hot_count[kMaxHot] = {};  // keys of each hot digit in this sub-tile so far
+  // Rows are ranked in groups: the LDS operations of a group are issued back
+  // to back and their results consumed together, so a wave waits for one LDS
+  // round trip per group, not per row.
+  // (Pairs hold their values in registers too and take smaller groups.)
+  constexpr int kGroup = kPairs ? ILGPU_HIP_SORT_PAIR_RANK_GROUP : ILGPU_HIP_SORT_RANK_GROUP;
+  static_assert(kGroup % 2 == 0, "ranks are packed in pairs");
 #pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    const uint32_t d = item_digit(j);
-    uint32_t rank = 0;
-    bool through_slot = true;
-    if constexpr (HOT) {
+  for (int j0 = 0; j0 < kItems; j0 += kGroup) {
+    uint32_t fetched[kGroup];   // what the LDS returned for the row
+    uint32_t offset[kGroup];    // added to it: lane index of a one-digit row
+    bool broadcast[kGroup];     // wave-uniform: take lane 0's result
 #pragma unroll
-      for (int h = 0; h < kMaxHot; ++h) {
-        if (hot[h] == kNoHotDigit) continue;  // wave-uniform
-        const bool is_hot = d == hot[h];
-        const uint64_t hot_lanes = __ballot(is_hot);
-        const uint32_t mine = (uint32_t)(hot_lanes >> (lane & ~(kSubLanes - 1))) & kSubLaneMask;
-        if (is_hot) {
-          rank = hot_count[h] + (uint32_t)__popc(mine & lower_lanes);
-          through_slot = false;
+    for (int g = 0; g < kGroup; ++g) {
+      const int j = j0 + g;
+      if (j >= kItems) break;
+      const uint32_t d = item_digit(j);
+      fetched[g] = 0;
+      offset[g] = 0;
+      broadcast[g] = false;
+      bool through_counter = true;
+      if constexpr (HOT) {
+#pragma unroll
+        for (int h = 0; h < kMaxHot; ++h) {
+          if (hot[h] == kNoHotDigit) continue;  // wave-uniform
+          const bool is_hot = d == hot[h];
+          const uint64_t hot_lanes = __ballot(is_hot);
+          if (is_hot) {
+            offset[g] = hot_count[h] + (uint32_t)mbcnt(hot_lanes);
+            through_counter = false;
+          }
+          hot_count[h] += (uint32_t)__popcll(hot_lanes);
         }
-        hot_count[h] += (uint32_t)__popc(mine);
-      }
-    }
-    if (through_slot) {
-      uint32_t* slot = my_slots + d;
-      // Keys that arrive in runs put one digit into whole rows of a sub-tile;
-      // the sixteen atomics of such a row would meet in one word and
-      // serialise (2^28 keys in runs of 1000: 0.92 ms per pass).  A row that
-      // is all one digit reads the count once (one address: a broadcast) and
-      // its first lane writes the new one (0.49 ms per pass on those keys,
-      // 0.7 % more on uniform ones).  Passes with dominant digits leave it
-      // out: the ballots above already took their frequent digits.
-      bool whole_row = false;
-      if constexpr (!HOT) {
-        const uint32_t row_digit = (uint32_t)__builtin_amdgcn_mov_dpp(
-            (int)d, 0x150 /* row_newbcast:0 */, 0xF, 0xF, false);
-        const uint64_t like_first = __ballot(d == row_digit);
-        whole_row = ((uint32_t)(like_first >> (lane & ~(kSubLanes - 1))) & kSubLaneMask) ==
-                    kSubLaneMask;
-      }
-      if (whole_row) {
-        const uint32_t before = __hip_atomic_load(slot, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_WORKGROUP) >> 16;
-        if (sub_lane == 0)
-          __hip_atomic_store(slot, (before + (uint32_t)kSubLanes) << 16, __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_WORKGROUP);
-        rank = before + (uint32_t)sub_lane;
       } else {
-        __hip_atomic_fetch_or(slot, lane_bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        const uint32_t both = __hip_atomic_load(slot, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_WORKGROUP);
-        const uint32_t peers = both & kSubLaneMask;
-        const uint32_t before = both >> 16;
-        const uint32_t below = (uint32_t)__popc(peers & lower_lanes);
-        if (below == 0)  // new count, mask cleared for the next row
-          __hip_atomic_store(slot, (before + (uint32_t)__popc(peers)) << 16,
-                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        rank = before + below;
+        // Keys that arrive in runs put one digit into whole rows of a
+        // sub-tile; the 64 atomics of such a row would meet in one word and
+        // serialise.  In a row that is all one digit only lane 0 adds (the
+        // whole row at once) and the others take its result plus their lane
+        // index.  Passes with dominant digits leave the check out: the
+        // ballots above already took their frequent digits.
+        const uint32_t row_digit = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+        broadcast[g] = __ballot(d == row_digit) == ~0ull;
+        if (broadcast[g]) {
+          offset[g] = (uint32_t)lane;
+          through_counter = lane == 0;
+        }
       }
+      if (through_counter)
+        fetched[g] = __hip_atomic_fetch_add(my_counters + d,
+                                            broadcast[g] ? (uint32_t)kSubLanes : 1u,
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    if (j % 2 == 0) packed[j / 2] = rank;
-    else packed[j / 2] |= rank << 16;
-    // Rows chain through LDS anyway.  Pin the packed rank here: left alone,
-    // the compiler sinks the rank arithmetic of all rows to where the ranks
-    // are used and keeps two live registers per key until then.
-    asm volatile("" : "+v"(packed[j / 2]));
+#pragma unroll
+    for (int g = 0; g < kGroup; ++g) {
+      const int j = j0 + g;
+      if (j >= kItems) break;
+      uint32_t rank = fetched[g];
+      if constexpr (!HOT) {
+        if (broadcast[g]) rank = (uint32_t)__builtin_amdgcn_readfirstlane((int)rank);
+      }
+      rank += offset[g];
+      if (j % 2 == 0) packed[j / 2] = rank;
+      else packed[j / 2] |= rank << 16;
+    }
+    // Pin the packed ranks here: left alone, the compiler sinks the rank
+    // arithmetic of all rows to where the ranks are used and keeps two live
+    // registers per key until then.
+#pragma unroll
+    for (int g = 0; g < kGroup; g += 2)
+      if (j0 + g < kItems) asm volatile("" : "+v"(packed[(j0 + g) / 2]));
   }
   if constexpr (HOT) {
 #pragma unroll
-    for (int h = 0; h < kMaxHot; ++h)  // these slots are untouched so far: still zero
-      if (hot[h] != kNoHotDigit && sub_lane == 0) my_slots[hot[h]] = hot_count[h] << 16;
+    for (int h = 0; h < kMaxHot; ++h)  // these counters are untouched so far: still zero
+      if (hot[h] != kNoHotDigit && lane == 0) my_counters[hot[h]] = hot_count[h];
   }
   __syncthreads();
 
@@ -483,7 +499,7 @@ __device__ __forceinline__ void sort_tile(
   uint32_t* tile_status = status + (int64_t)tile * kRadix;
   if (tid < kRadix) {
 #pragma unroll
-    for (int s = 0; s < kSubTiles; ++s) count += s_slot[s * kRadix + tid] >> 16;
+    for (int s = 0; s < kSubTiles; ++s) count += s_counter[s * kRadix + tid];
     __hip_atomic_store(&tile_status[tid],
                        tile == 0 ? status_prefix(count) : status_aggregate(count),
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -509,8 +525,8 @@ __device__ __forceinline__ void sort_tile(
       uint32_t run = digit_start;
 #pragma unroll
       for (int s = 0; s < kSubTiles; ++s) {
-        const uint32_t t = s_slot[s * kRadix + tid] >> 16;
-        s_slot[s * kRadix + tid] = run;
+        const uint32_t t = s_counter[s * kRadix + tid];
+        s_counter[s * kRadix + tid] = run;
         run += t;
       }
     }
@@ -523,12 +539,12 @@ __device__ __forceinline__ void sort_tile(
   }
   __syncthreads();
 
-  // Tile-local position of every key; afterwards the slots are dead and the
-  // same LDS bytes stage the keys in digit order.
+  // Tile-local position of every key; afterwards the counters are dead and
+  // the same LDS bytes stage the keys in digit order.
 #pragma unroll
   for (int j = 0; j < kItems; j += 2) {
-    const uint32_t p0 = my_slots[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
-    const uint32_t p1 = my_slots[item_digit(j + 1)] + (packed[j / 2] >> 16);
+    const uint32_t p0 = my_counters[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
+    const uint32_t p1 = my_counters[item_digit(j + 1)] + (packed[j / 2] >> 16);
     packed[j / 2] = p0 | (p1 << 16);
     if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
   }
@@ -591,7 +607,8 @@ __device__ __forceinline__ void sort_tile(
       dst_keys[g] = k;
       if constexpr (kPairs) gpos[j] = g;
     }
-    if (j % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+    constexpr int kWriteGroup = kPairs ? ILGPU_HIP_SORT_PAIR_WRITE_GROUP : ILGPU_HIP_SORT_WRITE_GROUP;
+    if (j % kWriteGroup == kWriteGroup - 1) __builtin_amdgcn_sched_barrier(0);
   }
 
   if constexpr (kPairs) {
@@ -659,7 +676,7 @@ void onesweep_kernel(
   // between a tile's ticket and the publication of its digit counts is what
   // every later tile's look-back waits for.  (Drawing it earlier, to load the
   // next keys during the write-out, measured 3 to 12 % slower.)  The key loads
-  // fly while the ranking slots are cleared.
+  // fly while the ranking counters are cleared.
   while (true) {
     if (tid == 0) s_tile = (int)atomicAdd(ticket, 1u);
     __syncthreads();  // also: the previous tile's staged keys have been read
@@ -667,32 +684,69 @@ void onesweep_kernel(
     if (tile >= num_tiles) break;
     const int64_t tile_base = (int64_t)tile * kTile;
     const int valid = valid_keys(tile);
-    K key[kItems];
-    if (valid == kTile) load_tile_keys<KEY_BYTES, kItems, true>(src_keys, tile_base, valid, first_local, key);
-    else load_tile_keys<KEY_BYTES, kItems, false>(src_keys, tile_base, valid, first_local, key);
-    {  // clear the ranking slots
-      uint4* z = reinterpret_cast<uint4*>(s_stage);
-      for (int i = tid; i < TileCfg::kSlotBytes / 16; i += kSortBlock)
-        z[i] = make_uint4(0u, 0u, 0u, 0u);
-    }
-    __syncthreads();
-    if (hot[0] == kNoHotDigit) {
-      if (valid == kTile) {
-        sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, true, false>(
-            key, dst_keys, src_vals, dst_vals, tile_base, kTile, tile, pass, xf,
-            excl, status, make_index, s_stage, s_global_off, s_scan, hot);
-      } else {
-        sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false, false>(
-            key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
-            excl, status, make_index, s_stage, s_global_off, s_scan, hot);
+    // Three instantiations of the tile code: full tiles with and without
+    // dominant digits, and the tail tile (bounds-checked; the dominant-digit
+    // form serves it either way: without such digits every key goes through
+    // the counters).  Each loads its keys itself, so that the loads, the
+    // clearing of the counters and the ranking are one straight line and the
+    // rows are ranked as their keys arrive.
+    auto run = [&](auto full, auto with_hot) {
+      constexpr bool kFull = decltype(full)::value;
+      constexpr bool kHot = decltype(with_hot)::value;
+      K key[kItems];
+      load_tile_keys<KEY_BYTES, kItems, kFull>(src_keys, tile_base, valid, first_local, key);
+      {  // clear the ranking counters
+        uint4* z = reinterpret_cast<uint4*>(s_stage);
+        for (int i = tid; i < TileCfg::kCounterBytes / 16; i += kSortBlock)
+          z[i] = make_uint4(0u, 0u, 0u, 0u);
       }
-    } else {
-      // The tail tile takes the same path: FULL only saves bounds checks.
-      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, false, true>(
-          key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf,
-          excl, status, make_index, s_stage, s_global_off, s_scan, hot);
-    }
+      __syncthreads();
+      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot>(
+          key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl, status,
+          make_index, s_stage, s_global_off, s_scan, hot);
+    };
+    if (valid != kTile) run(std::false_type{}, std::true_type{});
+    else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
+    else run(std::true_type{}, std::true_type{});
   }
+}
+
+// ---- device check of the LDS property the ranking rests on -------------------
+// Every wave keeps 256 counters and plays `rows` ranking rows on pseudo-random
+// digits drawn from `distinct` values: one returning LDS add per lane, then the
+// rank a lane got is compared with the rank memory order demands (count before
+// the row + lanes below it with the same digit, from eight ballots).  Lanes
+// served out of order are counted into *mismatches.
+__global__ __launch_bounds__(kSortBlock) void lds_atomic_order_kernel(
+    int rows, uint32_t distinct, uint64_t seed, unsigned long long* mismatches) {
+  __shared__ uint32_t s_counter[(kSortBlock / kWaveSize) * kRadix];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < (kSortBlock / kWaveSize) * kRadix; i += kSortBlock) s_counter[i] = 0u;
+  __syncthreads();
+  const int lane = tid & (kWaveSize - 1);
+  uint32_t* mine = s_counter + (tid / kWaveSize) * kRadix;
+  unsigned long long wrong = 0;
+  for (int r = 0; r < rows; ++r) {
+    uint64_t z = seed + ((uint64_t)blockIdx.x << 40) + ((uint64_t)r << 12) + (uint64_t)tid;
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    const uint32_t d = (uint32_t)(z % distinct) * ((uint32_t)kRadix / distinct);
+    uint64_t peers = ~0ull;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const bool bit = ((d >> b) & 1u) != 0;
+      const uint64_t m = __ballot(bit);
+      peers &= bit ? m : ~m;
+    }
+    const uint32_t before =
+        __hip_atomic_load(mine + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t rank =
+        __hip_atomic_fetch_add(mine + d, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (rank != before + (uint32_t)mbcnt(peers)) ++wrong;
+  }
+  if (wrong != 0) atomicAdd(mismatches, wrong);
 }
 
 // ---- finish ----------------------------------------------------------------
@@ -935,6 +989,20 @@ int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
 }
 
 }  // namespace
+
+int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches) {
+  int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(mismatches), 2);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  const int blocks = device_cu_count() * 4;  // every CU busy with several blocks
+  const uint32_t distinct[] = {1u, 2u, 4u, 16u, 64u, 256u};
+  for (int i = 0; i < 6; ++i) {
+    hipLaunchKernelGGL(lds_atomic_order_kernel, dim3((unsigned)blocks), dim3(kSortBlock), 0,
+                       stream, rows, distinct[i], 0x1234ull + (uint64_t)i,
+                       reinterpret_cast<unsigned long long*>(mismatches));
+    ILGPU_HIP_CHECK(hipGetLastError());
+  }
+  return ILGPU_HIP_SUCCESS;
+}
 
 int64_t radix_sort_max_length() { return kMaxSortLength; }
 

@@ -166,6 +166,19 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void *keys,
                                    int32_t flags, int32_t value_source,
                                    void *temp, int64_t temp_bytes);
 
+/* Device self-check of the one hardware property the sort's ranking relies
+ * on beyond the programming model: the lanes of ONE returning LDS atomic
+ * instruction that meet in one address are served in ascending lane order
+ * (this is what makes a pass stable at one LDS operation per key).  It has no
+ * counterpart in the reference; its place there is taken by the group-wide
+ * scans of RadixSortKernel1 (RadixSortExtensions.cs:700-705).  Plays `rows`
+ * (1 .. 2^20) ranking rows per wave on every compute unit for six digit
+ * distributions and stores the number of lanes found out of order in
+ * mismatches[0] (device memory, 8-byte aligned): 0 on gfx950.  Stream-ordered,
+ * allocates nothing. */
+int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
+                                            int32_t rows, int64_t *mismatches);
+
 /* ---- scan ---------------------------------------------------------------
  * Replaces: Scan<T,TStrideIn,TStrideOut> delegates made by CreateScan(kind)
  * (ScanExtensions.cs:52-61, 930-959) and ComputeScanTempStorageSize (:158-170).

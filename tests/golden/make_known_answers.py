@@ -15,6 +15,12 @@ library), so the vectors are independent of everything they are used to check:
   histogram HistogramTests.tt:42-103 (1..1024 into 64 / 256 bins by v % bins)
             and the overflow case :149-189
   transform TransformerExtensionTests.tt:66-134
+  float key order  RadixSortOperations.tt:77-93, 122-123 evaluated literally,
+            with C#'s integer promotions, on raw bit patterns of Half, float and
+            double keys (signed zeros, subnormals, infinities, NaNs, neighbours
+            in the last mantissa bit, negative values): no reference test sorts
+            such keys, so the expectation is the formula itself worked out with
+            Python integers, and a stable sort on the resulting key
 
 Run from the repository root:  python tests/golden/make_known_answers.py
 """
@@ -36,8 +42,78 @@ def sequence(start, step, n, bits, signed):
     return [wrap(start + i * step, bits, signed) for i in range(n)]
 
 
-def main():
+def csharp_float_sort_key(raw, bits):
+    """ExtractRadixBits of Ascending{Half,Float,Double} over all NumBits,
+    RadixSortOperations.tt:81-89, on the raw bit pattern `raw` of the key.
+
+    Half: Interop.FloatAsInt(Half) is a ushort (Interop.cs:171); `~` promotes it
+    to a 32-bit int, the (uint) cast binds before `>>`, so the shift is a
+    logical one of 0xFFFFxxxx by 15: bits 1..16 of the mask are always set and
+    bit 0 is the inverted sign.  float/double: `~` stays unsigned, the shift by
+    NumBits-1 leaves only the inverted sign in bit 0.  The sort's passes read
+    bits 0..NumBits-1 of `bits` two at a time (RadixSortExtensions.cs:1276-1334),
+    so the key is `bits` modulo 2^NumBits.
+    """
+    if bits == 16:
+        promoted = (-raw - 1) % (1 << 32)           # (uint)~(int)ushort
+        ones = promoted >> 15
+    else:
+        ones = ((-raw - 1) % (1 << bits)) >> (bits - 1)
+    sign_mask = 1 << (bits - 1)
+    return (raw ^ (sign_mask | ones)) % (1 << bits)
+
+
+def stable_order(keys):
+    # insertion into buckets by key, ties in input order
+    return [i for _, i in sorted((k, i) for i, k in enumerate(keys))]
+
+
+FLOAT_PATTERNS = {
+    # +0 -0 1 -1 2 -2 .5 -.5, smallest subnormals, infinities, NaNs (quiet,
+    # negative quiet, signalling), largest finite values, neighbours of +-1 in
+    # the last mantissa bit, and duplicates of 1, -1 and -0 (stability)
+    "float16": (16, [0x3C00, 0x4000, 0xBC00, 0xC000, 0x3800, 0xB800, 0x0000, 0x8000, 0x0001,
+                     0x8001, 0x7C00, 0xFC00, 0x7E00, 0xFE00, 0x7C01, 0x7BFF, 0xFBFF, 0x3C01,
+                     0xBC01, 0x3C00, 0xBC00, 0x8000, 0x3BFF, 0xBBFF]),
+    "float32": (32, [0x3F800000, 0x40000000, 0xBF800000, 0xC0000000, 0x3F000000, 0xBF000000,
+                     0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x7F800000, 0xFF800000,
+                     0x7FC00000, 0xFFC00000, 0x7F800001, 0x7F7FFFFF, 0xFF7FFFFF, 0x3F800001,
+                     0xBF800001, 0x3F800000, 0xBF800000, 0x80000000, 0x3F7FFFFF, 0xBF7FFFFF,
+                     0xC2F6E979, 0xC2F6E97A, 0xC47A0000, 0xC47A0000]),
+    "float64": (64, [0x3FF0000000000000, 0x4000000000000000, 0xBFF0000000000000,
+                     0xC000000000000000, 0x3FE0000000000000, 0xBFE0000000000000,
+                     0x0000000000000000, 0x8000000000000000, 0x0000000000000001,
+                     0x8000000000000001, 0x7FF0000000000000, 0xFFF0000000000000,
+                     0x7FF8000000000000, 0xFFF8000000000000, 0x7FF0000000000001,
+                     0x7FEFFFFFFFFFFFFF, 0xFFEFFFFFFFFFFFFF, 0x3FF0000000000001,
+                     0xBFF0000000000001, 0x3FF0000000000000, 0xBFF0000000000000,
+                     0x8000000000000000, 0x3FEFFFFFFFFFFFFF, 0xBFEFFFFFFFFFFFFF,
+                     0xC05EDD2F1A9FBE77, 0xC05EDD2F1A9FBE76, 0xC08F400000000000,
+                     0xC08F400000000000]),
+}
+
+
+def float_key_cases():
     cases = []
+    for name, (bits, raw) in FLOAT_PATTERNS.items():
+        mask = (1 << bits) - 1
+        asc_keys = [csharp_float_sort_key(r, bits) for r in raw]
+        for descending in (False, True):
+            # Descending*: every extracted digit is complemented (:122-123),
+            # i.e. the whole key is.
+            keys = [(~k) & mask for k in asc_keys] if descending else asc_keys
+            order = stable_order(keys)
+            cases.append({"op": "sort_float_bits", "dtype": name, "descending": descending,
+                          "input_bits": raw, "expected_bits": [raw[i] for i in order]})
+            cases.append({"op": "sort_pairs_float_bits", "dtype": name,
+                          "descending": descending, "input_bits": raw,
+                          "expected_bits": [raw[i] for i in order],
+                          "expected_index_values": order})
+    return cases
+
+
+def main():
+    cases = float_key_cases()
     for name, (bits, signed) in INT_TYPES.items():
         for n in SIZES:
             asc = sequence(0, 1, n, bits, signed)

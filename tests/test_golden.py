@@ -25,8 +25,24 @@ def by_op(op):
 
 
 def test_golden_file_covers_every_primitive():
-    assert OPS == ["histogram", "reduce", "scan", "sort", "sort_pairs", "transform"]
+    assert OPS == ["histogram", "reduce", "scan", "sort", "sort_float_bits", "sort_pairs",
+                   "sort_pairs_float_bits", "transform"]
     assert len(CASES) > 300
+    # Half, float and double keys, both orders, keys-only and pairs
+    assert len(by_op("sort_float_bits")) == 6 and len(by_op("sort_pairs_float_bits")) == 6
+
+
+_UINT_OF = {"float16": np.uint16, "float32": np.uint32, "float64": np.uint64}
+
+
+def float_keys(bits, dtype):
+    """Raw bit patterns of a golden case as an array of the float type."""
+    return np.array(bits, dtype=_UINT_OF[dtype]).view(np.dtype(dtype))
+
+
+def same_bits(got, bits, dtype):
+    return np.array_equal(np.ascontiguousarray(got).view(_UINT_OF[dtype]),
+                          np.array(bits, dtype=_UINT_OF[dtype]))
 
 
 # ------------------------------------------------------------------ CPU oracle
@@ -38,6 +54,38 @@ def test_oracle_sort_against_golden():
         k, v = O.radix_sort_pairs(arr(c["input"], c["dtype"]), arr(c["values"], c["dtype"]))
         assert np.array_equal(k, arr(c["expected"], c["dtype"]))
         assert np.array_equal(v, arr(c["expected_values"], c["dtype"]))
+
+
+def test_oracle_float_key_order_against_golden():
+    # The Half, float and double branches of the oracle's ascending_bits
+    # against the hand evaluation of RadixSortOperations.tt:81-89, 122-123
+    # (tests/golden/make_known_answers.py: Python integers only).
+    for c in by_op("sort_float_bits"):
+        got = O.radix_sort(float_keys(c["input_bits"], c["dtype"]), descending=c["descending"])
+        assert same_bits(got, c["expected_bits"], c["dtype"]), (c["dtype"], c["descending"])
+    for c in by_op("sort_pairs_float_bits"):
+        keys = float_keys(c["input_bits"], c["dtype"])
+        k, v = O.radix_sort_pairs(keys, np.arange(keys.size, dtype=np.uint32),
+                                  descending=c["descending"])
+        assert same_bits(k, c["expected_bits"], c["dtype"]), (c["dtype"], c["descending"])
+        assert v.tolist() == c["expected_index_values"], (c["dtype"], c["descending"])
+
+
+def test_half_key_example_worked_by_hand():
+    # Half keys: raw ^ (0xFFFE | !sign).  Positive values have every bit
+    # flipped (they follow the negative ones, in DEscending order), negative
+    # ones all but bit 0.
+    case = [c for c in by_op("sort_float_bits")
+            if c["dtype"] == "float16" and not c["descending"]][0]
+    assert 0x3C00 ^ 0xFFFF == 0xC3FF and 0xBC00 ^ 0xFFFE == 0x43FE
+    data = np.array([1, 2, -1, -2, .5, -.5], dtype=np.float16)
+    got = O.radix_sort(data)
+    assert got.tolist() == [-2, -1, -.5, 2, 1, .5]
+    # the golden case holds the same six values in that relative order
+    six = [b for b in case["expected_bits"] if b in (0x3C00, 0x4000, 0xBC00, 0xC000, 0x3800,
+                                                       0xB800)]
+    assert [x for i, x in enumerate(six) if x not in six[:i]] == [0xC000, 0xBC00, 0xB800,
+                                                                    0x4000, 0x3C00, 0x3800]
 
 
 _SCAN_OPS = {"add": O.OP_ADD, "max": O.OP_MAX, "min": O.OP_MIN}
@@ -83,6 +131,27 @@ def test_library_against_golden():
         torch.cuda.synchronize()
         assert np.array_equal(k.numpy(), arr(c["expected"], c["dtype"]))
         assert np.array_equal(v.numpy(), arr(c["expected_values"], c["dtype"]))
+    for c in by_op("sort_float_bits"):
+        d = D.from_numpy(float_keys(c["input_bits"], c["dtype"]))
+        capi.radix_sort_keys(d, descending=c["descending"])
+        torch.cuda.synchronize()
+        assert same_bits(d.numpy(), c["expected_bits"], c["dtype"]), \
+            ("sort", c["dtype"], c["descending"])
+    for c in by_op("sort_pairs_float_bits"):
+        keys = float_keys(c["input_bits"], c["dtype"])
+        k = D.from_numpy(keys)
+        v = D.zeros(keys.size, np.uint32)
+        capi.radix_sort_pairs(k, v, descending=c["descending"], values_from_index=True)
+        torch.cuda.synchronize()
+        assert same_bits(k.numpy(), c["expected_bits"], c["dtype"]), ("pairs", c["dtype"])
+        assert v.numpy().tolist() == c["expected_index_values"], ("pairs", c["dtype"])
+        # the same values handed in as a view
+        k = D.from_numpy(keys)
+        v = D.from_numpy(np.arange(keys.size, dtype=np.uint64))
+        capi.radix_sort_pairs(k, v, descending=c["descending"])
+        torch.cuda.synchronize()
+        assert same_bits(k.numpy(), c["expected_bits"], c["dtype"])
+        assert v.numpy().tolist() == c["expected_index_values"]
     ops = {"add": capi.OP_ADD, "max": capi.OP_MAX, "min": capi.OP_MIN}
     for c in by_op("scan"):
         x = arr(c["input"], c["dtype"])
