@@ -26,7 +26,8 @@ LIB_PATH = os.environ.get(
 
 # ilgpu_hip_status
 SUCCESS, ERROR_NULL_VIEW, ERROR_OUT_OF_RANGE, ERROR_NOT_SUPPORTED, \
-    ERROR_UNALIGNED_TEMP, ERROR_RUNTIME = range(6)
+    ERROR_UNALIGNED_TEMP, ERROR_RUNTIME, ERROR_STATIC_LIMIT = range(7)
+SCAN_STATIC_MAX_BYTES = 1 << 30
 # ilgpu_hip_type
 I8, I16, I32, I64, U8, U16, U32, U64, F16, F32, F64 = range(11)
 # ilgpu_hip_op / scan kind / flags / value source / locator
@@ -45,7 +46,7 @@ EXPORTS = [
     "ilgpu_hip_radix_sort_temp_bytes_strided",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
     "ilgpu_hip_selftest_lds_atomic_order",
-    "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan",
+    "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan", "ilgpu_hip_scan_static",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
     "ilgpu_hip_unique_temp_bytes", "ilgpu_hip_unique", "ilgpu_hip_initialize",
     "ilgpu_hip_sequence", "ilgpu_hip_reorder",
@@ -98,6 +99,7 @@ _ERRORS = {
     ERROR_NOT_SUPPORTED: NotSupportedError,
     ERROR_UNALIGNED_TEMP: InvalidOperationError,
     ERROR_RUNTIME: HipRuntimeError,
+    ERROR_STATIC_LIMIT: NotSupportedError,
 }
 
 _lib: Optional[ctypes.CDLL] = None
@@ -134,6 +136,8 @@ def lib() -> ctypes.CDLL:
         L.ilgpu_hip_scan_temp_bytes.argtypes = [i64, i32, p64]
         L.ilgpu_hip_scan.argtypes = [vp, vp, i64, i64, vp, i64, i64, i32, i32,
                                      i32, vp, i64]
+        L.ilgpu_hip_scan_static.argtypes = [vp, vp, i64, i64, vp, i64, i64, i32, i32, i32]
+        L.ilgpu_hip_scan_static.restype = i32
         L.ilgpu_hip_reduce_temp_bytes.argtypes = [i64, i32, p64]
         L.ilgpu_hip_unique_temp_bytes.argtypes = [i64, i32, p64]
         L.ilgpu_hip_unique.argtypes = [vp, vp, i64, i32, vp, i64, vp, i64]
@@ -322,6 +326,14 @@ def scan(inp: DeviceArray, out: DeviceArray, temp: Optional[DeviceArray] = None,
     check(lib().ilgpu_hip_scan(
         _stream_ptr(stream), inp.ptr, inp.length, inp.stride, out.ptr,
         out.length, out.stride, inp.type_code, op, kind, temp.ptr, temp.nbytes))
+
+
+def scan_static(inp: DeviceArray, out: DeviceArray, *, op: int = OP_ADD,
+                kind: int = SCAN_INCLUSIVE, stream=None) -> None:
+    """The scan on the library's static scratch: no temp, no allocation."""
+    check(lib().ilgpu_hip_scan_static(
+        _stream_ptr(stream), inp.ptr, inp.length, inp.stride, out.ptr,
+        out.length, out.stride, inp.type_code, op, kind))
 
 
 def reduce_temp_bytes(n: int, dtype) -> int:

@@ -145,6 +145,9 @@ const char* ilgpu_hip_status_string(int32_t status) {
     case ILGPU_HIP_ERROR_NOT_SUPPORTED: return "not supported";
     case ILGPU_HIP_ERROR_UNALIGNED_TEMP: return "unaligned temp allocation";
     case ILGPU_HIP_ERROR_RUNTIME: return "HIP runtime error";
+    case ILGPU_HIP_ERROR_STATIC_LIMIT:
+      return "input exceeds what the library's static scratch serves "
+             "(ilgpu_hip_scan_static: 1 GiB of input)";
     default: return "unknown status";
   }
 }
@@ -304,6 +307,28 @@ int32_t ilgpu_hip_scan(ilgpu_hip_stream_t stream, const void* in,
   if (rc != ILGPU_HIP_SUCCESS) return rc;
   return launch_scan(static_cast<hipStream_t>(stream), in, in_stride, out,
                      out_stride, in_length, elem_type, op, kind, temp);
+}
+
+int32_t ilgpu_hip_scan_static(ilgpu_hip_stream_t stream, const void* in,
+                              int64_t in_length, int64_t in_stride, void* out,
+                              int64_t out_length, int64_t out_stride,
+                              int32_t elem_type, int32_t op, int32_t kind) {
+  /* The checks of ilgpu_hip_scan, in its order; no temp to check. */
+  if (!scan_reduce_type(elem_type) || !valid_op(op) ||
+      (kind != ILGPU_HIP_SCAN_INCLUSIVE && kind != ILGPU_HIP_SCAN_EXCLUSIVE))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (!valid_view(in, in_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (!valid_view(out, out_length)) return ILGPU_HIP_ERROR_NULL_VIEW;
+  if (out_length < in_length) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (in_length > INT32_MAX) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int eb = elem_size(elem_type);
+  if (in_stride < 1 || out_stride < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (!aligned_to(in, eb) || !aligned_to(out, eb))
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (in_length * eb > ILGPU_HIP_SCAN_STATIC_MAX_BYTES)
+    return ILGPU_HIP_ERROR_STATIC_LIMIT;
+  return launch_scan_static(static_cast<hipStream_t>(stream), in, in_stride, out,
+                            out_stride, in_length, elem_type, op, kind);
 }
 
 /* ---- reduce ------------------------------------------------------------ */

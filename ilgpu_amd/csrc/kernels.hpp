@@ -20,6 +20,12 @@ int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
                     void* out, int64_t out_stride, int64_t n, int32_t type,
                     int32_t op, int32_t kind, void* temp);
 
+// Same on the library's static scratch (no temp view, no allocation); inputs of
+// more than ILGPU_HIP_SCAN_STATIC_MAX_BYTES return ILGPU_HIP_ERROR_STATIC_LIMIT.
+int32_t launch_scan_static(hipStream_t stream, const void* in, int64_t in_stride,
+                           void* out, int64_t out_stride, int64_t n, int32_t type,
+                           int32_t op, int32_t kind);
+
 // histogram.hip
 int32_t launch_histogram(hipStream_t stream, const void* in, int64_t n,
                          int64_t in_stride, int32_t in_type, void* bins,

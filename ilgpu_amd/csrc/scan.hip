@@ -24,6 +24,9 @@
 // Each tile's words sit in a 128-byte line of their own.
 //
 // Algorithmic HBM traffic: 2 * n * sizeof(T) bytes (status: 128 B/tile).
+#include <atomic>
+#include <mutex>
+
 #include "kernels.hpp"
 
 namespace ilgpu_hip {
@@ -684,6 +687,52 @@ int32_t launch_scan(hipStream_t stream, const void* in, int64_t in_stride,
     case ILGPU_HIP_F64: return launch_op<double>(stream, in, in_stride, out, out_stride, n, op, kind, temp);
     default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
+}
+
+// ---- scan on the library's own scratch ---------------------------------------
+// For callers that cannot allocate or carry a temp view: the tile states of one
+// scan live in a device array that is part of the library's code object.  It is
+// sized for kStaticScanTiles tiles (1 GiB of input); every call on a GPU shares
+// that GPU's copy, so calls that overlap in time on one GPU race.
+constexpr int64_t kSmallestTileBytes =
+    (int64_t)kBlock * 16 * (scan_vecs<uint32_t>() < scan_vecs<uint64_t>() ? scan_vecs<uint32_t>()
+                                                                           : scan_vecs<uint64_t>());
+constexpr int64_t kStaticScanTiles = ILGPU_HIP_SCAN_STATIC_MAX_BYTES / kSmallestTileBytes;
+constexpr int64_t kStaticScratchBytes = kHeaderBytes + kStaticScanTiles * kStatusBytes;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+}  // namespace
+
+int32_t launch_scan_static(hipStream_t stream, const void* in, int64_t in_stride,
+                           void* out, int64_t out_stride, int64_t n, int32_t type,
+                           int32_t op, int32_t kind) {
+  // The tiles of this call must fit the array: scan_temp_bytes() minus the
+  // alignment slack a caller's temp needs (the array is aligned itself).
+  if (scan_temp_bytes(n, elem_size(type)) - 256 > kStaticScratchBytes)
+    return ILGPU_HIP_ERROR_STATIC_LIMIT;
+  int device = -1;
+  ILGPU_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  // Every GPU holds its own copy of the array at its own address; the array's
+  // name is no device address on the host.  Looked up once per device.
+  void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ptr = g_scratch_ptr[device].load(std::memory_order_relaxed);
+    if (ptr == nullptr) {
+      ILGPU_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+      if (ptr == nullptr) return ILGPU_HIP_ERROR_RUNTIME;
+      g_scratch_ptr[device].store(ptr, std::memory_order_release);
+    }
+  }
+  // launch_scan clears the ticket and the status lines it will use with a fill
+  // kernel (the array keeps the previous call's contents) and hands `ptr` to
+  // the scan kernel as it does with a caller's temp.
+  return launch_scan(stream, in, in_stride, out, out_stride, n, type, op, kind, ptr);
 }
 
 int64_t unique_temp_bytes(int64_t n, int elem_bytes) {

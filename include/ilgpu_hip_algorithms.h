@@ -53,8 +53,11 @@ typedef enum ilgpu_hip_status {
   ILGPU_HIP_ERROR_NOT_SUPPORTED = 3,  /* NotSupportedException */
   ILGPU_HIP_ERROR_UNALIGNED_TEMP = 4, /* InvalidOperationException
                                          (TempViewManager.cs:98-106) */
-  ILGPU_HIP_ERROR_RUNTIME = 5         /* a HIP call failed; see
+  ILGPU_HIP_ERROR_RUNTIME = 5,        /* a HIP call failed; see
                                          ilgpu_hip_last_runtime_error() */
+  ILGPU_HIP_ERROR_STATIC_LIMIT = 6    /* NotSupportedException: the input is
+                                         larger than the library's static
+                                         scratch serves (ilgpu_hip_scan_static) */
 } ilgpu_hip_status;
 
 /* Element types: NumericTypes of TypeInformation.ttinclude:94-121. */
@@ -195,6 +198,27 @@ int32_t ilgpu_hip_scan(ilgpu_hip_stream_t stream, const void *in,
                        int64_t out_length, int64_t out_stride,
                        int32_t elem_type, int32_t op, int32_t kind, void *temp,
                        int64_t temp_bytes);
+
+/* The same scan without a temp view, for callers that cannot allocate device
+ * memory or carry a temp buffer: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose Scan delegates always take an ArrayView<int> temp,
+ * ScanExtensions.cs:52-61).  The tile states live in a device array inside the
+ * library (1 MiB + 256 bytes per GPU, held until the process ends), so
+ *  - the input may hold at most ILGPU_HIP_SCAN_STATIC_MAX_BYTES bytes
+ *    (in_length * element size); more returns ILGPU_HIP_ERROR_STATIC_LIMIT;
+ *  - every call on one GPU uses that GPU's array: calls that overlap in time on
+ *    the same GPU (two streams, two threads) race and must be serialised by the
+ *    caller;
+ *  - the call allocates nothing and clears what it needs with a fill kernel
+ *    (no memset node), so it may be captured into a graph; the first call on a
+ *    device looks up the array's address and should be made outside a capture.
+ * Arguments, checks and results are those of ilgpu_hip_scan. */
+#define ILGPU_HIP_SCAN_STATIC_MAX_BYTES (1ll << 30)
+int32_t ilgpu_hip_scan_static(ilgpu_hip_stream_t stream, const void *in,
+                              int64_t in_length, int64_t in_stride, void *out,
+                              int64_t out_length, int64_t out_stride,
+                              int32_t elem_type, int32_t op, int32_t kind);
 
 /* ---- reduce -------------------------------------------------------------
  * Replaces: Reduction<T,TStride> delegates made by CreateReduction and the
