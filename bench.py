@@ -81,35 +81,46 @@ def kernel_stats(capi, name):
     return launches, (total_ms / launches if launches else 0.0)
 
 
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3
-# (FETCH_SIZE and WRITE_SIZE in separate runs of this script, each scaled by
-# what the same counter reads for a 1 GiB device copy: 2.00 and 1.00).  A
-# counter run cannot be nested inside this script, so the figure of the
-# committed profile is reported for the workload it was taken on.
-MEASURED_TRAFFIC_BYTES = {
-    # (kernel, log2 n): bytes per launch
-    ("onesweep_kernel<4,0>", 28): 2.392e9,
-}
-# The same for the other workloads at their default sizes, keyed by bench name.
-MEASURED_EXTRA_TRAFFIC_BYTES = {
-    "scan_exclusive_add_i32_2^28": 2.178e9,
-    "reduce_add_f32_2^28": 1.074e9,
-    "histogram_u8_256bins_2^30": 1.075e9,
-    "histogram_i32_4096bins_2^28": 1.086e9,
-    "radix_sort_pairs_u64_u32_2^27": 3.644e9,
-    "unique_i32_all_distinct_2^28": 2.176e9,
-    "sequence_i32_2^28": 1.074e9,
-    "initialize_i32_2^28": 1.074e9,
-    "transform_negate_i32_2^28": 2.147e9,
-    "transform_i32_to_i64_2^28": 3.221e9,
-    "reorder_u32_random_permutation_2^28": 3.638e10,
-}
+# HBM bytes per launch of each workload's dominant kernel come from rocprofv3
+# counter runs of this script (FETCH_SIZE and WRITE_SIZE in separate runs, each
+# scaled by what the same counter reads for a 1 GiB device copy).  A counter
+# run cannot be nested inside this script, so the figures are kept in
+# profiles/hbm_traffic.json together with the SHA-256 of the kernel source they
+# were measured on; a figure whose source has changed since is not reported.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+CSRC = os.path.join(ROOT, "ilgpu_amd", "csrc")
 
 
-def roofline(achieved_gbs, traffic=None):
-    return {"bound": "hbm", "achieved": round(achieved_gbs, 1),
-            "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic}
+def source_digest(file_name):
+    import hashlib
+    with open(os.path.join(CSRC, file_name), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def measured_traffic(workload, default_size):
+    """(bytes per launch or None, provenance) for a bench workload."""
+    if not default_size or not os.path.exists(TRAFFIC_FILE):
+        return None, None
+    with open(TRAFFIC_FILE) as f:
+        table = json.load(f)
+    entry = table.get("workloads", {}).get(workload)
+    if entry is None:
+        return None, None
+    source = {"file": "profiles/hbm_traffic.json", "kernel_source": entry["source"],
+              "measured_on_sha256": entry["sha256"]}
+    if source_digest(entry["source"]) != entry["sha256"]:
+        source["stale"] = "kernel source changed since the counters were read"
+        return None, source
+    return entry["bytes_per_launch"], source
+
+
+def roofline(achieved_gbs, traffic=None, traffic_source=None):
+    r = {"bound": "hbm", "achieved": round(achieved_gbs, 1),
+         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic}
+    if traffic_source is not None:
+        r["traffic_source"] = traffic_source
+    return r
 
 
 def main():
@@ -150,7 +161,8 @@ def main():
 
     log(f"[bench] radix sort: {W} warm-up + {K} timed steps")
     ms, wall = timer.run(restore, sort, K, W)
-    ms_per_step = float(np.mean(ms))
+    ms_per_step = float(np.median(ms))   # median of the K timed steps
+    mean_ms_per_step = float(np.mean(ms))
     gkeys = n / (ms_per_step * 1e-3) / 1e9
 
     # Same K steps again with the library's per-kernel event timing enabled.
@@ -209,6 +221,8 @@ def main():
         "steps": K,
         "warmup": W,
         "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_statistic": "median",
+        "mean_ms_per_step": round(mean_ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -219,8 +233,8 @@ def main():
                                "(SplitMix64 seed 0x123456789ABCDEF0)",
                    "n": n, "passes_executed": passes,
                    "algorithmic_bytes_per_key": 4 * (2 * passes + 1)},
-        "roofline": dict(roofline(pass_gbs, MEASURED_TRAFFIC_BYTES.get(
-                             ("onesweep_kernel<4,0>", args.log2n))),
+        "roofline": dict(roofline(pass_gbs, *measured_traffic(
+                             "radix_sort_u32_uniform_2^28", args.log2n == 28)),
                          kernel="onesweep_kernel<4,0>",
                          bytes_per_launch=pass_bytes,
                          avg_launch_ms=round(pass_ms, 4),
@@ -258,14 +272,14 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
         timer.run(prepare, fn, K, 0)
         launches, k_ms = kernel_stats(capi, kernel)
         capi.profile_enable(False)
-        t = float(np.mean(ms))
+        t = float(np.median(ms))
         kb = kernel_bytes if kernel_bytes is not None else algo_bytes
         k_gbs = kb / (k_ms * 1e-3) / 1e9 if k_ms else 0.0
         entry = {"ms_per_step": round(t, 4),
+                 "mean_ms_per_step": round(float(np.mean(ms)), 4),
                  "algorithmic_gbs": round(algo_bytes / (t * 1e-3) / 1e9, 1),
                  "frac_of_hbm_peak": round(algo_bytes / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                 "roofline": dict(roofline(k_gbs, MEASURED_EXTRA_TRAFFIC_BYTES.get(name)
-                                           if args.log2n == 28 else None),
+                 "roofline": dict(roofline(k_gbs, *measured_traffic(name, args.log2n == 28)),
                                   kernel=kernel, avg_launch_ms=round(k_ms, 4))}
         out[name] = entry
         log(f"[bench] {name}: {t:.3f} ms/step, {entry['algorithmic_gbs']:.0f} GB/s "
@@ -338,6 +352,12 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
               lambda: capi.histogram(d_in, bins, ov), n28 * 4.0, "histogram")
     expect = torch.bincount(g.to(torch.int64), minlength=4096)
     e["verified"] = bool(np.array_equal(bins.numpy().astype(np.int64), expect.cpu().numpy()))
+    if cpu_on:
+        m = 1 << min(28, args.log2n)
+        s = g[:m].cpu().numpy()
+        t0 = time.perf_counter(); O.histogram(s, np.zeros(4096, dtype=np.int32)); dt = time.perf_counter() - t0
+        e["cpu_baseline"] = {"value": round(m * 4.0 / dt / 1e9, 3), "unit": "GB/s", "cores": 1,
+                             "kind": "port", "sample": f"2^{int(np.log2(m))} keys, {dt:.2f} s"}
     del g, d_in, expect
 
     # RadixSortPairs of 2^27 uint64 keys with uint32 index payload
@@ -358,6 +378,23 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
     ties = wk[1:] == wk[:-1]
     ok_stable = bool((wv[1:][ties] > wv[:-1][ties]).all().item())
     e["verified"] = ok_sorted and ok_perm and ok_stable
+    if cpu_on:
+        m = 1 << min(23, args.log2n)
+        sk = k64[:m].cpu().numpy().view(np.uint64)
+        t0 = time.perf_counter()
+        rk, rv = O.radix_sort_pairs(sk, np.arange(m, dtype=np.uint32))
+        dt = time.perf_counter() - t0
+        e["cpu_baseline"] = {"value": round(m / dt / 1e9, 5), "unit": "Gpairs/s", "cores": 1,
+                             "kind": "port",
+                             "sample": f"first 2^{int(np.log2(m))} pairs, {dt:.1f} s (32 passes of "
+                                       "2 bits over 16-byte key/value records)"}
+        # the same sample through the GPU path must agree bit for bit
+        gk, gv = D.from_numpy(sk), D.zeros(m, np.uint32)
+        capi.radix_sort_pairs(gk, gv, values_from_index=True)
+        torch.cuda.synchronize()
+        e["verified"] = e["verified"] and bool(np.array_equal(gk.numpy(), rk)) and \
+            bool(np.array_equal(gv.numpy(), rv))
+        del sk, rk, rv, gk, gv
     del k64, wk, wv, dk, dv, temp, flip
 
     # Skewed sorts: Zipf(1.1) over 2^16 values, and all keys equal
@@ -371,7 +408,7 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
         capi.profile_enable(True)
         timer.run(lambda: work.copy_(src), lambda: capi.radix_sort_keys(keys, temp), 1, 0)
         capi.profile_enable(False)
-        t = float(np.mean(ms))
+        t = float(np.median(ms))
         o64 = work.to(torch.int64) & 0xFFFFFFFF
         ok = bool((o64[1:] >= o64[:-1]).all().item()) and \
             int(o64.sum().item()) == int((src.to(torch.int64) & 0xFFFFFFFF).sum().item())
@@ -383,6 +420,19 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
                      "algorithmic_gbs": round(algo / (t * 1e-3) / 1e9, 1),
                      "frac_of_hbm_peak": round(algo / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "verified": ok}
+        if cpu_on:
+            m = 1 << min(25, args.log2n)
+            sample = src[:m].cpu().numpy().view(np.uint32)
+            t0 = time.perf_counter(); ref = O.radix_sort(sample); dt = time.perf_counter() - t0
+            out[name]["cpu_baseline"] = {
+                "value": round(m / dt / 1e9, 5), "unit": "Gkeys/s", "cores": 1, "kind": "port",
+                "sample": f"first 2^{int(np.log2(m))} keys, {dt:.1f} s (the CPU path runs all 16 "
+                          "passes whatever the keys)"}
+            dsample = D.from_numpy(sample)
+            capi.radix_sort_keys(dsample)
+            torch.cuda.synchronize()
+            out[name]["verified"] = ok and bool(np.array_equal(dsample.numpy(), ref))
+            del sample, ref, dsample
         log(f"[bench] {name}: {t:.3f} ms/step, {out[name]['gkeys_per_s']} Gkeys/s")
         del work, keys, temp, o64, src
 

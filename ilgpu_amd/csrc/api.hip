@@ -14,21 +14,30 @@ namespace ilgpu_hip {
 
 namespace {
 thread_local int32_t g_last_runtime_error = 0;
-std::atomic<int> g_cu_count{0};
+std::atomic<int> g_cu_count[kMaxCachedDevices];
 }  // namespace
 
 void set_last_runtime_error(hipError_t e) { g_last_runtime_error = (int32_t)e; }
 
+int current_device() {
+  int dev = -1;
+  return hipGetDevice(&dev) == hipSuccess ? dev : -1;
+}
+
 int device_cu_count() {
-  int cached = g_cu_count.load(std::memory_order_relaxed);
-  if (cached > 0) return cached;
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
+  const int dev = current_device();
+  const bool cacheable = dev >= 0 && dev < kMaxCachedDevices;
+  if (cacheable) {
+    const int cached = g_cu_count[dev].load(std::memory_order_relaxed);
+    if (cached > 0) return cached;
+  }
+  int cus = 0;
+  if (dev < 0 ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) !=
           hipSuccess ||
       cus <= 0)
     cus = 256;
-  g_cu_count.store(cus, std::memory_order_relaxed);
+  if (cacheable) g_cu_count[dev].store(cus, std::memory_order_relaxed);
   return cus;
 }
 

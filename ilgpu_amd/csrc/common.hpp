@@ -26,7 +26,10 @@ void set_last_runtime_error(hipError_t e);
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 inline int64_t div_up(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// Number of compute units of the current device (cached per process).
+// The current device's index (-1 if the runtime cannot tell) and its number of
+// compute units (cached per device).
+constexpr int kMaxCachedDevices = 64;
+int current_device();
 int device_cu_count();
 
 // Optional per-kernel timing (the library's counterpart of ILGPU's
@@ -179,15 +182,20 @@ template <typename T> struct Functor<T, ILGPU_HIP_OP_ADD> {
 // Math.Max / Math.Min of the reference's MaxFloat/MinDouble... functors
 // (ScanReduceOperations.tt:36-72, IntrinsicMath.cs:111-112, 207-208): a NaN
 // operand wins (the first one if both are), and -0.0 < +0.0.  The hardware
-// maximum and minimum already order the signed zeros that way and return the
-// other operand for a NaN, so only the NaN selection is added.
+// maximum and minimum return the other operand for a NaN; what they return
+// for (+0, -0) is not specified by the builtin, so equal operands (that is
+// the two zeros, or identical values) are told apart by their sign bit.
 template <typename T> __device__ __forceinline__ T fp_hw_max(T a, T b) {
-  if constexpr (sizeof(T) == 4) return __builtin_fmaxf(a, b);
-  else return __builtin_fmax(a, b);
+  T m;
+  if constexpr (sizeof(T) == 4) m = __builtin_fmaxf(a, b);
+  else m = __builtin_fmax(a, b);
+  return a == b ? (fp_signbit(a) ? b : a) : m;
 }
 template <typename T> __device__ __forceinline__ T fp_hw_min(T a, T b) {
-  if constexpr (sizeof(T) == 4) return __builtin_fminf(a, b);
-  else return __builtin_fmin(a, b);
+  T m;
+  if constexpr (sizeof(T) == 4) m = __builtin_fminf(a, b);
+  else m = __builtin_fmin(a, b);
+  return a == b ? (fp_signbit(a) ? a : b) : m;
 }
 template <typename T> struct Functor<T, ILGPU_HIP_OP_MAX> {
   static __device__ __forceinline__ T identity() { return Limits<T>::lowest(); }

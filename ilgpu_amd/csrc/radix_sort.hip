@@ -55,6 +55,9 @@ constexpr int kMaxPasses = 8;
 #ifndef ILGPU_HIP_SORT_ITEMS8
 #define ILGPU_HIP_SORT_ITEMS8 18
 #endif
+#ifndef ILGPU_HIP_SORT_PAIR_ITEMS3
+#define ILGPU_HIP_SORT_PAIR_ITEMS3 16
+#endif
 #ifndef ILGPU_HIP_SORT_LOOKBACK
 #define ILGPU_HIP_SORT_LOOKBACK 4
 #endif
@@ -125,7 +128,7 @@ constexpr int items_per_thread(int key_bytes, int value_bytes) {
   if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS8 : ILGPU_HIP_SORT_ITEMS;
   if (value_bytes == 16) return 8;
   const int registers = (key_bytes == 8 ? 2 : 1) + (value_bytes == 8 ? 2 : 1);
-  return registers == 2 ? 20 : registers == 3 ? 16 : 14;
+  return registers == 2 ? 20 : registers == 3 ? ILGPU_HIP_SORT_PAIR_ITEMS3 : 14;
 }
 constexpr int tile_keys(int key_bytes, int value_bytes) {
   return kSortBlock * items_per_thread(key_bytes, value_bytes);
@@ -335,8 +338,9 @@ __device__ __forceinline__ void load_tile_keys(
 }
 
 // Waves per SIMD the pass kernel is compiled for: two blocks of eight waves
-// per CU.  That bounds a thread at 128 registers (28 keys, 14 registers of
-// packed ranks and the values of a pair fit) and a block at 80 KiB of LDS.
+// per CU.  That bounds a thread at 128 registers (36 keys and 18 registers of
+// packed ranks in a keys-only sort; fewer items when values ride along) and a
+// block at 80 KiB of LDS (the 36-key tile stages 72 KiB).
 #ifndef ILGPU_HIP_SORT_WAVES_PER_EU
 #define ILGPU_HIP_SORT_WAVES_PER_EU 4
 #endif
@@ -705,9 +709,14 @@ void onesweep_kernel(
           key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl, status,
           make_index, s_stage, s_global_off, s_scan, hot);
     };
+#ifdef ILGPU_HIP_SORT_NO_FULL_HOT
+    if (hot[0] != kNoHotDigit || valid != kTile) run(std::false_type{}, std::true_type{});
+    else run(std::true_type{}, std::false_type{});
+#else
     if (valid != kTile) run(std::false_type{}, std::true_type{});
     else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
     else run(std::true_type{}, std::true_type{});
+#endif
   }
 }
 
@@ -878,15 +887,19 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
     if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true>;
   }
-  // Resident blocks per CU of this instantiation: asked once per process and
+  // Resident blocks per CU of this instantiation: asked once per device and
   // kernel (the query costs microseconds, which small sorts would feel).
-  static std::atomic<int> cached_per_cu[2] = {{0}, {0}};
-  int per_cu = cached_per_cu[float_keys ? 1 : 0].load(std::memory_order_relaxed);
+  static std::atomic<int> cached_per_cu[kMaxCachedDevices][2];
+  const int device = current_device();
+  std::atomic<int>* cached =
+      device >= 0 && device < kMaxCachedDevices ? &cached_per_cu[device][float_keys ? 1 : 0]
+                                                : nullptr;
+  int per_cu = cached ? cached->load(std::memory_order_relaxed) : 0;
   if (per_cu == 0) {
     ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
         &per_cu, pass_kernel, kSortBlock, 0));
     if (per_cu < 1) per_cu = 1;
-    cached_per_cu[float_keys ? 1 : 0].store(per_cu, std::memory_order_relaxed);
+    if (cached) cached->store(per_cu, std::memory_order_relaxed);
   }
   int64_t grid = (int64_t)cus * per_cu;
   if (grid > L.tiles) grid = L.tiles;

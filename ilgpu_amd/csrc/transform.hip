@@ -54,7 +54,10 @@ __device__ __forceinline__ S apply_transformer(S v, int op, int64_t factor) {
     switch (op) {
       case ILGPU_HIP_TRANSFORM_NEGATE: return (S)(U)(0u - (U)v);
       case ILGPU_HIP_TRANSFORM_BIT_COMPLEMENT: return (S)(U)~(U)v;
-      case ILGPU_HIP_TRANSFORM_MULTIPLY: return (S)(U)((U)v * (U)(uint64_t)factor);
+      // In 64 bits: 8- and 16-bit operands would be promoted to int, whose
+      // product can overflow (0xFFFF * 0xFFFF); the low bits are the same.
+      case ILGPU_HIP_TRANSFORM_MULTIPLY:
+        return (S)(U)((uint64_t)(U)v * (uint64_t)factor);
       default: return v;
     }
   }

@@ -20,10 +20,14 @@
 #include <cstdint>
 #include <functional>
 #include <limits>
+#include <map>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <type_traits>
+#include <typeindex>
+#include <typeinfo>
 #include <vector>
 
 #include "../../include/ilgpu_hip_algorithms.h"
@@ -217,9 +221,21 @@ class Accelerator {
   }
   void Synchronize() { CheckHip(hipDeviceSynchronize()); }
   int Device() const { return device_; }
+  // Objects the algorithms keep per accelerator (cached delegates and their
+  // scratch), created on first use and released with the accelerator, the way
+  // ILGPU caches loaded kernels per accelerator.
+  template <typename TKey, typename TObject>
+  std::shared_ptr<TObject> GetOrCreateCached(const std::function<std::shared_ptr<TObject>()>& make) {
+    std::lock_guard<std::mutex> lock(cache_mutex_);
+    std::shared_ptr<void>& slot = cache_[std::type_index(typeid(TKey))];
+    if (!slot) slot = make();
+    return std::static_pointer_cast<TObject>(slot);
+  }
  private:
   int device_;
   AcceleratorStream default_;
+  std::mutex cache_mutex_;
+  std::map<std::type_index, std::shared_ptr<void>> cache_;
 };
 
 // ---- functors ------------------------------------------------------------------
@@ -574,6 +590,27 @@ std::unique_ptr<ScanProvider> CreateScanProvider(Accelerator& a, LongIndex1D dat
 template <typename T, typename TStride>
 using Reduction = std::function<void(AcceleratorStream&, ArrayView1D<T, TStride>, ArrayView<T>)>;
 
+// The scratch of the native reduction (partial results of the first kernel),
+// one buffer per stream: the reference's delegate has no hidden state and may
+// be invoked on several streams at once (ReductionExtensions.cs:135-167), so
+// invocations on different streams must not share partials.  A stream's buffer
+// is allocated at the first invocation on that stream and kept.
+class ReductionScratch {
+ public:
+  ReductionScratch(Accelerator& accelerator, int64_t ints) : accelerator_(accelerator), ints_(ints) {}
+  ArrayView<int32_t> For(AcceleratorStream& stream) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    std::unique_ptr<MemoryBuffer1D<int32_t>>& slot = by_stream_[stream.StreamPtr()];
+    if (!slot) slot = accelerator_.Allocate1D<int32_t>(ints_);
+    return slot->View();
+  }
+ private:
+  Accelerator& accelerator_;
+  int64_t ints_;
+  std::mutex mutex_;
+  std::map<hipStream_t, std::unique_ptr<MemoryBuffer1D<int32_t>>> by_stream_;
+};
+
 // CreateReduction (:135-167).  The delegate owns the scratch the native
 // kernels need (the reference's delegate has no temp argument).
 template <typename T, typename TStride, typename TReduction>
@@ -583,30 +620,37 @@ Reduction<T, TStride> CreateReduction(Accelerator& accelerator) {
   int64_t bytes = 0;
   HipAlgorithmsException::ThrowIfFailed(
       ilgpu_hip_reduce_temp_bytes(1, TypeCode<T>::value, &bytes));
-  std::shared_ptr<MemoryBuffer1D<int32_t>> scratch(
-      accelerator.Allocate1D<int32_t>(BytesToInts(bytes)).release());
-  return [scratch](AcceleratorStream& stream, ArrayView1D<T, TStride> input,
-                   ArrayView<T> output) {
+  auto scratch_by_stream = std::make_shared<ReductionScratch>(accelerator, BytesToInts(bytes));
+  return [scratch_by_stream](AcceleratorStream& stream, ArrayView1D<T, TStride> input,
+                             ArrayView<T> output) {
     if (!input.IsValid()) throw ArgumentNullException("input");
     if (input.Length() < 1) throw ArgumentOutOfRangeException("input");
     if (!output.IsValid()) throw ArgumentNullException("output");
     if (output.Length() < 1) throw ArgumentOutOfRangeException("output");
+    const ArrayView<int32_t> scratch = scratch_by_stream->For(stream);
     HipAlgorithmsException::ThrowIfFailed(
         ilgpu_hip_reduce(stream.StreamPtr(), input.LoadEffectiveAddressAsPtr(), input.Length(),
                          input.Stride().Stride(),
                          TypeCode<T>::value, TReduction::Op,
                          output.LoadEffectiveAddressAsPtr(), output.Length(),
-                         scratch->View().LoadEffectiveAddressAsPtr(),
-                         scratch->View().Length() * 4),
+                         scratch.LoadEffectiveAddressAsPtr(), scratch.Length() * 4),
         "input");
   };
 }
 
-// Reduce into a view (:180-190).
+// Reduce into a view (:180-190).  The delegate (and with it the scratch) is
+// made once per accelerator, element type and functor and reused: the call
+// stays stream-ordered and allocates only the first time a stream is seen.
 template <typename T, typename TReduction>
 void Reduce(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<T> input,
             ArrayView<T> output) {
-  CreateReduction<T, Stride1D::Dense, TReduction>(accelerator)(stream, input, output);
+  using Delegate = Reduction<T, Stride1D::Dense>;
+  struct CacheKey {};  // one per instantiation
+  auto reduction = accelerator.GetOrCreateCached<CacheKey, Delegate>([&accelerator]() {
+    return std::make_shared<Delegate>(
+        CreateReduction<T, Stride1D::Dense, TReduction>(accelerator));
+  });
+  (*reduction)(stream, input, output);
 }
 // Reduce returning the value (:204-216): synchronises the stream.
 template <typename T, typename TReduction>

@@ -479,6 +479,46 @@ static void ReduceErrors(Accelerator& accl) {
   EXPECT_THROW(reduce(s, in->View(), ArrayView<float>()), ArgumentNullException);
 }
 
+// One delegate invoked on two streams at once: the reference's delegate has no
+// hidden state (ReductionExtensions.cs:135-167), so neither may ours.  Large
+// inputs keep both reductions in flight together; every invocation must give
+// its own input's sum.
+static void ReduceOnTwoStreams(Accelerator& accl) {
+  auto reduce = CreateReduction<int64_t, Stride1D::Dense, SRO::AddInt64>(accl);
+  const int length = 1 << 22;
+  std::vector<int64_t> a((size_t)length), b((size_t)length);
+  int64_t sumA = 0, sumB = 0;
+  for (int i = 0; i < length; ++i) {
+    a[i] = i % 7;
+    b[i] = -(int64_t)(i % 5) - 1;
+    sumA += a[i];
+    sumB += b[i];
+  }
+  auto inA = accl.Allocate1D<int64_t>(a);
+  auto inB = accl.Allocate1D<int64_t>(b);
+  auto outA = accl.Allocate1D<int64_t>(1);
+  auto outB = accl.Allocate1D<int64_t>(1);
+  auto s1 = accl.CreateStream();
+  auto s2 = accl.CreateStream();
+  for (int round = 0; round < 20; ++round) {
+    reduce(*s1, inA->View(), outA->View());
+    reduce(*s2, inB->View(), outB->View());
+    reduce(*s1, inA->View(), outA->View());
+    reduce(*s2, inB->View(), outB->View());
+  }
+  s1->Synchronize();
+  s2->Synchronize();
+  CHECK(outA->GetAsArray1D()[0] == sumA);
+  CHECK(outB->GetAsArray1D()[0] == sumB);
+  // the cached delegate behind Reduce(accelerator, stream, input, output)
+  Reduce<int64_t, SRO::AddInt64>(accl, *s1, inA->View(), outB->View());
+  Reduce<int64_t, SRO::AddInt64>(accl, *s2, inB->View(), outA->View());
+  s1->Synchronize();
+  s2->Synchronize();
+  CHECK(outB->GetAsArray1D()[0] == sumA);
+  CHECK(outA->GetAsArray1D()[0] == sumB);
+}
+
 // ---- HistogramTests -----------------------------------------------------------
 template <typename T, typename TBin> void HistogramTests(Accelerator& accl) {
   using Modulo = HistogramOperations::ModuloBinOperation;
@@ -583,6 +623,7 @@ int main(int argc, char** argv) {
     RUN((ReduceTests<float, SRO::AddFloat>(accl, 1000)));
     RUN((ReduceTests<double, SRO::MaxDouble>(accl, 1000)));
     RUN(ReduceErrors(accl));
+    RUN(ReduceOnTwoStreams(accl));
     RUN((HistogramTests<int32_t, int32_t>(accl)));
     RUN((HistogramTests<uint8_t, uint32_t>(accl)));
     RUN((HistogramTests<int64_t, int64_t>(accl)));

@@ -49,7 +49,7 @@ def test_sort_2p28_uniform_u32_sorted_and_same_multiset():
     assert torch.equal(again, work)
 
 
-def test_sort_2p28_descending_is_reverse_of_ascending():
+def test_sort_2p28_zipf_against_its_value_counts_and_descending_is_the_reverse():
     import torch
     n = 1 << 28
     note("sort 2^28 zipf u32 ascending vs descending")
@@ -59,6 +59,61 @@ def test_sort_2p28_descending_is_reverse_of_ascending():
     capi.radix_sort_keys(wrap(desc, np.uint32), descending=True)
     torch.cuda.synchronize()
     assert torch.equal(torch.flip(desc, [0]), asc)
+    # Against the source, independently of the library: the keys take 2^16
+    # values, so the sorted array is fully determined by the value counts of
+    # the input (torch.bincount): value v fills [start[v], start[v] + count[v]).
+    a = u32(asc)
+    counts = torch.bincount(u32(src), minlength=1 << 16)
+    assert counts.numel() == 1 << 16
+    assert bool((a[1:] >= a[:-1]).all().item())
+    assert torch.equal(torch.bincount(a, minlength=1 << 16), counts)
+    starts = torch.cumsum(counts, 0) - counts
+    present = torch.nonzero(counts).flatten()
+    assert torch.equal(a[starts[present]], present)                       # first key of every run
+    assert torch.equal(a[starts[present] + counts[present] - 1], present)  # and its last
+
+
+def test_sort_2p28_all_equal_keys_runs_no_pass_and_leaves_the_input():
+    import torch
+    n = 1 << 28
+    note("sort 2^28 all-equal u32")
+    src = torch.full((n,), -559038737, dtype=torch.int32, device="cuda:0")   # 0xDEADBEEF
+    work = src.clone()
+    temp = capi.temp_buffer(capi.radix_sort_temp_bytes(n, np.uint32))
+    capi.profile_enable(True)
+    capi.radix_sort_keys(wrap(work, np.uint32), temp)
+    torch.cuda.synchronize()
+    launches, pass_ms = capi.profile_query("sort_onesweep")
+    _, hist_ms = capi.profile_query("sort_histogram")
+    capi.profile_enable(False)
+    assert torch.equal(work, src)
+    # every digit is the same for all keys, so all four pass launches return at once
+    assert launches == 4 and pass_ms < 0.25 * hist_ms, (launches, pass_ms, hist_ms)
+    # one key differs: its pass and only its pass runs, and the odd key moves to the front
+    work[n // 3] = -559038737 - 1                                            # 0xDEADBEEE
+    capi.radix_sort_keys(wrap(work, np.uint32), temp)
+    torch.cuda.synchronize()
+    assert int(work[0].item()) == -559038738 and bool((work[1:] == -559038737).all().item())
+
+
+def test_histogram_2p28_i32_4096_bins_against_bincount():
+    import torch
+    n = 1 << 28
+    note("histogram 2^28 i32 -> 4096 bins")
+    g = datagen.gaussian_mixture_i32_torch(n)
+    bins, ov = D.zeros(4096, np.int32), D.zeros(1, np.int32)
+    capi.histogram(wrap(g, np.int32), bins, ov)
+    torch.cuda.synchronize()
+    expect = torch.zeros(4096, dtype=torch.int64, device="cuda:0")
+    for lo in range(0, n, 1 << 26):                       # chunked: bincount widens to int64
+        expect += torch.bincount(g[lo: lo + (1 << 26)].to(torch.int64), minlength=4096)
+    assert np.array_equal(bins.numpy().astype(np.int64), expect.cpu().numpy())
+    assert int(expect.sum().item()) == n and ov.numpy()[0] == 0
+    # int64 bins and the modulo locator give the same counts (all keys are in [0, 4095])
+    wide = D.zeros(4096, np.int64)
+    capi.histogram(wrap(g, np.int32), wide, locator=capi.LOCATOR_MODULO)
+    torch.cuda.synchronize()
+    assert np.array_equal(wide.numpy(), expect.cpu().numpy())
 
 
 def test_pairs_2p27_u64_index_values_invert_the_sort():
