@@ -80,9 +80,16 @@ typedef enum ilgpu_hip_scan_kind {
 /* Sort flags.  DESCENDING selects the Descending* functor
  * (RadixSortOperations.tt:98-125).  By default floating-point keys are
  * ordered exactly as the reference's ExtractRadixBits orders them
- * (RadixSortOperations.tt:81-89, including what it does to negative values);
- * FLOAT_TOTAL_ORDER instead sorts them in IEEE-754 totalOrder and has no
- * counterpart in the reference. */
+ * (RadixSortOperations.tt:81-89), and that order is NOT numerically monotone:
+ * the mask meant to complement negative values comes from a logical shift of
+ * an unsigned pattern, so an "ascending" sort of float or double keys leaves
+ * the negative ones in ascending magnitude ([-0.5, -1, -2, 0.5, 1, 2]) and
+ * positive keys that differ only in the last mantissa bit swapped; for Half
+ * (whose bits are promoted to a 32-bit int before the shift) the negative
+ * keys are in numeric order and the positive ones in descending order
+ * ([-2, -1, -0.5, 2, 1, 0.5]).  FLOAT_TOTAL_ORDER instead sorts in IEEE-754
+ * totalOrder (-NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN), the
+ * numerically sorted result; it has no counterpart in the reference. */
 enum {
   ILGPU_HIP_SORT_DESCENDING = 1,
   ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER = 2
