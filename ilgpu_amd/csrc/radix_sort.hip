@@ -709,14 +709,9 @@ void onesweep_kernel(
           key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl, status,
           make_index, s_stage, s_global_off, s_scan, hot);
     };
-#ifdef ILGPU_HIP_SORT_NO_FULL_HOT
-    if (hot[0] != kNoHotDigit || valid != kTile) run(std::false_type{}, std::true_type{});
-    else run(std::true_type{}, std::false_type{});
-#else
     if (valid != kTile) run(std::false_type{}, std::true_type{});
     else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
     else run(std::true_type{}, std::true_type{});
-#endif
   }
 }
 

@@ -606,6 +606,16 @@ def gpu_unique(values):
     return d.numpy()[:kept], d.numpy()[kept:], kept
 
 
+def test_lds_atomics_serve_the_lanes_of_an_instruction_in_lane_order():
+    # The hardware property the sort's ranking rests on (one returning LDS add per
+    # key, equal digits must come back in lane order): checked on every compute
+    # unit, under load, for six digit distributions.  Any lane served out of
+    # order would make a pass unstable, which the pair-sort tests would show too.
+    assert capi.selftest_lds_atomic_order(2048) == 0
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.selftest_lds_atomic_order(0)
+
+
 @pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
 @pytest.mark.parametrize("repeat", [1, 317, 1025])
 def test_unique_reference_cases(dtype, repeat):
