@@ -19,6 +19,7 @@
 
 #include <cstdint>
 #include <functional>
+#include <future>
 #include <limits>
 #include <map>
 #include <memory>
@@ -659,6 +660,18 @@ T Reduce(Accelerator& accelerator, AcceleratorStream& stream, ArrayView<T> input
   Reduce<T, TReduction>(accelerator, stream, input, output->View());
   stream.Synchronize();
   return output->GetAsArray1D()[0];
+}
+
+// ReduceAsync (:230-236, :302-309): Task.Run(() => Reduce(...)).  The stream
+// and the accelerator must outlive the future, as they must outlive the task
+// in the reference.
+template <typename T, typename TReduction>
+std::future<T> ReduceAsync(Accelerator& accelerator, AcceleratorStream& stream,
+                           ArrayView<T> input) {
+  return std::async(std::launch::async, [&accelerator, &stream, input]() {
+    CheckHip(hipSetDevice(accelerator.Device()));  // a new thread starts on device 0
+    return Reduce<T, TReduction>(accelerator, stream, input);
+  });
 }
 
 // ---- histogram (HistogramExtensions.cs, HistogramLaunchers.tt) -------------------

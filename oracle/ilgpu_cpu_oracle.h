@@ -12,8 +12,13 @@
  *                               sequences RadixSortExtensionTests.tt:37-131).
  *                               float/double >= 0 at integer values and constant -1:
  *                               pinned by the same sequences.  Negative floats,
- *                               adjacent positive floats and Half: PARITY UNPINNED
- *                               (restated as written, no reference test covers them).
+ *                               adjacent positive floats and Half: no reference test
+ *                               covers them; pinned by golden vectors worked out by
+ *                               hand from RadixSortOperations.tt:81-89, 122-123 with
+ *                               C#'s integer promotion rules, in Python integers only
+ *                               (tests/golden/make_known_answers.py, ops
+ *                               sort_float_bits and sort_pairs_float_bits: Half,
+ *                               float and double, both orders, keys and pairs).
  *   oracle_radix_sort[_pairs]   pinned against stable sort by extracted key.
  *   oracle_scan                 integers pinned against serial fold
  *                               (ScanExtensionTests.tt:286-305); floating point

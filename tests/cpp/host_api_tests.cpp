@@ -517,6 +517,11 @@ static void ReduceOnTwoStreams(Accelerator& accl) {
   s2->Synchronize();
   CHECK(outB->GetAsArray1D()[0] == sumA);
   CHECK(outA->GetAsArray1D()[0] == sumB);
+  // ReduceAsync (ReductionExtensions.cs:230-236): two tasks at once, one per stream
+  auto futureA = ReduceAsync<int64_t, SRO::AddInt64>(accl, *s1, inA->View());
+  auto futureB = ReduceAsync<int64_t, SRO::AddInt64>(accl, *s2, inB->View());
+  CHECK(futureA.get() == sumA);
+  CHECK(futureB.get() == sumB);
 }
 
 // ---- HistogramTests -----------------------------------------------------------

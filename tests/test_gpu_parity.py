@@ -353,8 +353,9 @@ def test_sort_integer_types_match_oracle(dtype, descending):
 @pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
 @pytest.mark.parametrize("descending", [False, True])
 def test_sort_float_types_match_reference_order(dtype, descending):
-    # Default float order = the reference's ExtractRadixBits as written
-    # (parity unpinned by reference tests for negative values; see the oracle).
+    # Default float order = the reference's ExtractRadixBits as written (no
+    # reference test has negative or Half keys; the oracle's transform is held
+    # by the hand-evaluated golden vectors of tests/test_golden.py).
     keys = random_float_bits(dtype, 30011, seed=3)
     assert bits_equal(gpu_sort(keys, descending=descending),
                       O.radix_sort(keys, descending=descending))
