@@ -283,6 +283,11 @@ int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
                                           mismatches);
 }
 
+int32_t ilgpu_hip_set_sort_lookback_spin_limit(int32_t polls) {
+  set_sort_lookback_spin_limit(polls);
+  return ILGPU_HIP_SUCCESS;
+}
+
 /* ---- scan -------------------------------------------------------------- */
 
 int32_t ilgpu_hip_scan_temp_bytes(int64_t n, int32_t elem_type,

@@ -72,6 +72,20 @@ constexpr int kMaxPasses = 8;
 #ifndef ILGPU_HIP_SORT_PAIR_WRITE_GROUP
 #define ILGPU_HIP_SORT_PAIR_WRITE_GROUP 4
 #endif
+// Tiles are handed out in chunks of consecutive tiles, one chunk at a time to
+// each of kTicketGroups groups of blocks (block b is in group b % 8: blocks are
+// dispatched round-robin over the eight XCDs, so a group is the blocks of one
+// XCD).  Neighbouring tiles write neighbouring runs; when they run on one XCD
+// the partially written lines between their runs merge in that XCD's L2.
+#ifndef ILGPU_HIP_SORT_MAX_CHUNK_SHIFT
+#define ILGPU_HIP_SORT_MAX_CHUNK_SHIFT 3
+#endif
+constexpr int kTicketGroups = 8;
+constexpr int kTicketStride = 32;          // words: one 128-byte line per group
+constexpr int kMaxChunkShift = ILGPU_HIP_SORT_MAX_CHUNK_SHIFT;
+// Polls of an empty status word before a look-back stops waiting for the tile
+// and counts its digit itself.
+constexpr uint32_t kDefaultSpinLimit = 4096;
 #ifndef ILGPU_HIP_SORT_WRITE_GROUP
 #define ILGPU_HIP_SORT_WRITE_GROUP 12
 #endif
@@ -349,12 +363,14 @@ __device__ __forceinline__ void load_tile_keys(
 template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT>
 __device__ __forceinline__ void sort_tile(
     typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
+    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys,
     typename KeyOf<KEY_BYTES>::type* __restrict__ dst_keys,
     const typename ValueOf<VALUE_BYTES>::type* __restrict__ src_vals,
     typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
     int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
     const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
-    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan, const uint32_t (&hot)[kMaxHot]) {
+    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan,
+    const uint32_t (&hot)[kMaxHot], uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
@@ -584,7 +600,21 @@ __device__ __forceinline__ void sort_tile(
 #pragma unroll
       for (int u = 0; u < kLookback; ++u) {
         if (done) continue;
+        uint32_t polls = 0;
         while (s[u] == 0u) {
+          if (polls++ >= spin_limit) {
+            // Nobody has published tile t - u: its owner may not be running.
+            // Count this thread's digit in that tile from the source keys (a
+            // full tile: it precedes this one) and go on as if the tile had
+            // published its own count.  Slow, and never needed while every
+            // group of blocks is resident.
+            const K* other = src_keys + (int64_t)(t - u) * TileCfg::kTile;
+            uint32_t c = 0;
+#pragma unroll 4
+            for (int i = 0; i < TileCfg::kTile; ++i) c += digit(other[i]) == (uint32_t)tid;
+            s[u] = status_aggregate(c);
+            break;
+          }
           __builtin_amdgcn_s_sleep(1);
           s[u] = __hip_atomic_load(&status[(int64_t)(t - u) * kRadix + tid],
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -645,7 +675,7 @@ void onesweep_kernel(
     typename ValueOf<VALUE_BYTES>::type* vals_b, int64_t n, int pass,
     KeyXform xf, const uint32_t* __restrict__ excl, uint32_t* status,
     uint32_t* ticket, const SortPlan* __restrict__ plan, int num_tiles,
-    int values_from_index) {
+    int values_from_index, int chunk_shift, uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
@@ -676,13 +706,26 @@ void onesweep_kernel(
     return remaining >= kTile ? kTile : (remaining > 0 ? (int)remaining : 0);
   };
 
+  // Tickets: group g (= blockIdx % 8) owns the chunks g, g + 8, g + 16, ... of
+  // 2^chunk_shift consecutive tiles and draws their tiles in order from its
+  // own counter.  Unlike a single counter this does not start tiles in index
+  // order across groups: a tile can find that a predecessor owned by another
+  // group has not been started, and if that group had no resident block it
+  // would wait for ever.  The look-back therefore never waits without bound:
+  // after spin_limit polls of an empty word it counts the tile's digit itself
+  // (sort_tile), so every block finishes whatever the other blocks do.
   // A block draws its next tile only when it is about to start it: the time
   // between a tile's ticket and the publication of its digit counts is what
   // every later tile's look-back waits for.  (Drawing it earlier, to load the
   // next keys during the write-out, measured 3 to 12 % slower.)  The key loads
   // fly while the ranking counters are cleared.
   while (true) {
-    if (tid == 0) s_tile = (int)atomicAdd(ticket, 1u);
+    if (tid == 0) {
+      const uint32_t g = blockIdx.x % (uint32_t)kTicketGroups;
+      const uint32_t k = atomicAdd(ticket + g * kTicketStride, 1u);
+      const uint32_t chunk = (k >> chunk_shift) * kTicketGroups + g;
+      s_tile = (int)((chunk << chunk_shift) + (k & ((1u << chunk_shift) - 1u)));
+    }
     __syncthreads();  // also: the previous tile's staged keys have been read
     const int tile = s_tile;
     if (tile >= num_tiles) break;
@@ -706,8 +749,8 @@ void onesweep_kernel(
       }
       __syncthreads();
       sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot>(
-          key, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl, status,
-          make_index, s_stage, s_global_off, s_scan, hot);
+          key, src_keys, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl,
+          status, make_index, s_stage, s_global_off, s_scan, hot, spin_limit);
     };
     if (valid != kTile) run(std::false_type{}, std::true_type{});
     else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
@@ -780,6 +823,8 @@ __global__ __launch_bounds__(256) void finish_kernel(
 }
 
 // ---- host side -------------------------------------------------------------
+std::atomic<uint32_t> g_spin_limit{kDefaultSpinLimit};
+
 struct TempLayout {
   int64_t alt_keys, alt_vals, excl, plan, zero_begin, hist, tickets, status,
       status_stride, total;
@@ -797,7 +842,7 @@ TempLayout make_layout(int64_t n, int key_bytes, int value_bytes) {
   L.plan = off; off += 256;
   L.zero_begin = off;
   L.hist = off; off += kMaxPasses * kRadix * 4;
-  L.tickets = off; off += 256;
+  L.tickets = off; off += kMaxPasses * kTicketGroups * kTicketStride * 4;
   L.status = off;
   L.status_stride = L.tiles * kRadix * 4;
   off += L.status_stride * key_bytes;  // one status array per pass
@@ -898,6 +943,11 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   }
   int64_t grid = (int64_t)cus * per_cu;
   if (grid > L.tiles) grid = L.tiles;
+  // Chunks as long as leave every block of the grid a tile of its own in the
+  // first round (short inputs: single tiles, handed out round-robin).
+  int chunk_shift = 0;
+  while (chunk_shift < kMaxChunkShift && (grid << (chunk_shift + 1)) <= L.tiles) ++chunk_shift;
+  const uint32_t spin_limit = g_spin_limit.load(std::memory_order_relaxed);
   for (int p = 0; p < passes; ++p) {
     uint32_t* status =
         reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
@@ -906,7 +956,8 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
       hipLaunchKernelGGL(pass_kernel,
                          dim3((unsigned)grid), dim3(kSortBlock), 0, stream,
                          keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
-                         status, tickets + p, plan, (int)L.tiles, from_index);
+                         status, tickets + p * kTicketGroups * kTicketStride, plan, (int)L.tiles,
+                         from_index, chunk_shift, spin_limit);
     }
     ILGPU_HIP_CHECK(hipGetLastError());
   }
@@ -997,6 +1048,10 @@ int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
 }
 
 }  // namespace
+
+void set_sort_lookback_spin_limit(int32_t polls) {
+  g_spin_limit.store(polls < 0 ? kDefaultSpinLimit : (uint32_t)polls, std::memory_order_relaxed);
+}
 
 int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches) {
   int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(mismatches), 2);

@@ -189,6 +189,18 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void *keys,
 int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
                                             int32_t rows, int64_t *mismatches);
 
+/* How long the look-back of a sort pass polls the status word of an earlier
+ * tile that has published nothing before it stops waiting and counts that
+ * tile's digit itself from the source keys (the sort's tiles are handed to
+ * fixed groups of blocks, so a tile may wait for one whose group has no
+ * resident block; with this bound every block finishes whatever the others
+ * do).  polls < 0 restores the default (4096); 0 makes every look-back that
+ * meets an empty word take the slow path at once, which is how the tests
+ * exercise it.  Process-wide, applies to sorts launched afterwards.  No
+ * counterpart in the reference (its passes are separate kernel launches,
+ * RadixSortExtensions.cs:1276-1334). */
+int32_t ilgpu_hip_set_sort_lookback_spin_limit(int32_t polls);
+
 /* ---- scan ---------------------------------------------------------------
  * Replaces: Scan<T,TStrideIn,TStrideOut> delegates made by CreateScan(kind)
  * (ScanExtensions.cs:52-61, 930-959) and ComputeScanTempStorageSize (:158-170).

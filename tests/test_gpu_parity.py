@@ -617,6 +617,38 @@ def test_lds_atomics_serve_the_lanes_of_an_instruction_in_lane_order():
         capi.selftest_lds_atomic_order(0)
 
 
+def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
+    # A pass hands its tiles to eight fixed groups of blocks, so a tile's
+    # look-back can meet a predecessor nobody has started; past a bound of polls
+    # it counts that tile's digit itself from the source keys.  With the bound
+    # at zero every empty status word takes that path; results must not change.
+    capi.set_sort_lookback_spin_limit(0)
+    try:
+        for dtype, n in [(np.uint32, 18432 * 40 + 77), (np.uint8, 300000), (np.int16, 400001),
+                         (np.uint64, 9216 * 33 + 5)]:
+            note("sort with zero spin limit", np.dtype(dtype).name, n)
+            keys = random_ints(dtype, n, seed=11)
+            assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+        keys = random_float_bits(np.float32, 500000, seed=12)
+        assert bits_equal(gpu_sort(keys, descending=True), O.radix_sort(keys, descending=True))
+        # pairs: few distinct keys, so stability decides the value order
+        keys = random_ints(np.uint32, 300000, seed=13, lo=0, hi=999)
+        values = np.arange(keys.size, dtype=np.uint64)
+        k, v = gpu_sort_pairs(keys, values)
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(k, keys[order]) and np.array_equal(v, values[order])
+        keys = random_ints(np.int64, 200000, seed=14)
+        values = random_ints(np.uint8, keys.size, seed=15)
+        k, v = gpu_sort_pairs(keys, values)
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(k, keys[order]) and np.array_equal(v, values[order])
+    finally:
+        capi.set_sort_lookback_spin_limit(-1)
+    # back on the default bound
+    keys = random_ints(np.uint32, 18432 * 40 + 77, seed=16)
+    assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+
+
 @pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
 @pytest.mark.parametrize("repeat", [1, 317, 1025])
 def test_unique_reference_cases(dtype, repeat):
