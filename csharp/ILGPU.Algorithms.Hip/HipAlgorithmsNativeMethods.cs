@@ -37,8 +37,8 @@ namespace ILGPU.Algorithms.Hip
             int keyType, int valueBytes, int flags, int valueSource, void* temp, long tempBytes);
         [DllImport(LibName)] internal static extern int ilgpu_hip_selftest_lds_atomic_order(
             IntPtr stream, int rows, long* mismatches);
-        [DllImport(LibName)] internal static extern int ilgpu_hip_set_sort_lookback_spin_limit(
-            int polls);
+        [DllImport(LibName)] internal static extern int ilgpu_hip_sort_set_parameter(
+            int parameter, int value);
 
         [DllImport(LibName)] internal static extern int ilgpu_hip_scan_temp_bytes(
             long n, int elemType, out long tempBytes);

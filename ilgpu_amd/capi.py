@@ -45,7 +45,7 @@ EXPORTS = [
     "ilgpu_hip_profile_query", "ilgpu_hip_radix_sort_temp_bytes",
     "ilgpu_hip_radix_sort_temp_bytes_strided",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
-    "ilgpu_hip_selftest_lds_atomic_order", "ilgpu_hip_set_sort_lookback_spin_limit",
+    "ilgpu_hip_selftest_lds_atomic_order", "ilgpu_hip_sort_set_parameter",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan", "ilgpu_hip_scan_static",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
     "ilgpu_hip_unique_temp_bytes", "ilgpu_hip_unique", "ilgpu_hip_initialize",
@@ -133,8 +133,8 @@ def lib() -> ctypes.CDLL:
             vp, vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, i64]
         L.ilgpu_hip_selftest_lds_atomic_order.argtypes = [vp, i32, vp]
         L.ilgpu_hip_selftest_lds_atomic_order.restype = i32
-        L.ilgpu_hip_set_sort_lookback_spin_limit.argtypes = [i32]
-        L.ilgpu_hip_set_sort_lookback_spin_limit.restype = i32
+        L.ilgpu_hip_sort_set_parameter.argtypes = [i32, i32]
+        L.ilgpu_hip_sort_set_parameter.restype = i32
         L.ilgpu_hip_scan_temp_bytes.argtypes = [i64, i32, p64]
         L.ilgpu_hip_scan.argtypes = [vp, vp, i64, i64, vp, i64, i64, i32, i32,
                                      i32, vp, i64]
@@ -317,10 +317,20 @@ def selftest_lds_atomic_order(rows: int = 256, *, stream=None) -> int:
     return int(out.numpy()[0])
 
 
+SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0
+SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1
+
+
+def sort_set_parameter(parameter: int, value: int) -> None:
+    """Process-wide sort parameter; a negative value restores the default.
+    LOOKBACK_SPIN_LIMIT: polls of an empty status word before a pass counts a
+    missing tile itself (0 = at once: exercises the slow path).
+    LARGE_BLOCK_MIN_TILES_PER_CU: 0 = always 1024-thread blocks, 2^31-1 = never."""
+    check(lib().ilgpu_hip_sort_set_parameter(parameter, value))
+
+
 def set_sort_lookback_spin_limit(polls: int) -> None:
-    """Polls of an empty status word before a sort pass counts a missing tile
-    itself; negative = default, 0 = at once (exercises the slow path)."""
-    check(lib().ilgpu_hip_set_sort_lookback_spin_limit(polls))
+    sort_set_parameter(SORT_PARAM_LOOKBACK_SPIN_LIMIT, polls)
 
 
 def scan_temp_bytes(n: int, dtype) -> int:

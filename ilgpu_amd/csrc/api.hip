@@ -283,8 +283,11 @@ int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
                                           mismatches);
 }
 
-int32_t ilgpu_hip_set_sort_lookback_spin_limit(int32_t polls) {
-  set_sort_lookback_spin_limit(polls);
+int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value) {
+  if (parameter != ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT &&
+      parameter != ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU)
+    return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  set_sort_parameter(parameter, value);
   return ILGPU_HIP_SUCCESS;
 }
 

@@ -50,9 +50,8 @@ int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
                               int64_t key_stride = 1, int64_t value_stride = 1);
 int64_t radix_sort_max_length();
 int32_t launch_radix_sort(hipStream_t stream, const SortArgs& args);
-// Polls of an empty look-back status word before a pass counts the missing
-// tile's digit itself; negative restores the default.
-void set_sort_lookback_spin_limit(int32_t polls);
+// ILGPU_HIP_SORT_PARAM_* (validated by the caller); negative = default.
+void set_sort_parameter(int32_t parameter, int32_t value);
 // Device check of the LDS behaviour the sort's ranking relies on: lanes of one
 // returning LDS atomic that share an address are served in lane order.
 // mismatches[0] (device) receives the number of lanes found out of order.

@@ -89,7 +89,18 @@ constexpr uint32_t kDefaultSpinLimit = 4096;
 #ifndef ILGPU_HIP_SORT_WRITE_GROUP
 #define ILGPU_HIP_SORT_WRITE_GROUP 12
 #endif
-constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;
+// Two block sizes.  Large inputs take 1024-thread blocks, one per compute unit:
+// twice the tile, so every digit's run is twice as long (it is run length that
+// the scattered writes pay for, pairs above all, whose tiles are short), and
+// half as many tiles to chain.  Smaller inputs take 512-thread blocks, two per
+// compute unit, which fill the GPU with fewer keys.
+constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;      // small inputs, and the self-test
+constexpr int kSortBlockLarge = 1024;
+// The large block is used from this many of its tiles per compute unit on
+// (measured crossovers: 2^28 / 2^27 u32 keys gain 3 % / 1 %, 2^26 lose 4 %;
+// pairs of u64 keys and u32 values gain 4 to 8 % from 2^23 pairs on).
+constexpr int kLargeMinTilesPerCuKeys = 10;
+constexpr int kLargeMinTilesPerCuPairs = 2;
 // Lanes that rank together (a sub-tile row): one wave.
 constexpr int kSubLanes = kWaveSize;
 constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
@@ -144,8 +155,8 @@ constexpr int items_per_thread(int key_bytes, int value_bytes) {
   const int registers = (key_bytes == 8 ? 2 : 1) + (value_bytes == 8 ? 2 : 1);
   return registers == 2 ? 20 : registers == 3 ? ILGPU_HIP_SORT_PAIR_ITEMS3 : 14;
 }
-constexpr int tile_keys(int key_bytes, int value_bytes) {
-  return kSortBlock * items_per_thread(key_bytes, value_bytes);
+constexpr int tile_keys(int key_bytes, int value_bytes, int block) {
+  return block * items_per_thread(key_bytes, value_bytes);
 }
 
 // How raw key bits map to unsigned bits that sort in the requested order.
@@ -326,12 +337,12 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 // checked on the device by ilgpu_hip_selftest_lds_atomic_order and, end to
 // end, by every stability test of the pair sorts.  With it the pass is stable
 // at one LDS operation per key and no cross-lane arithmetic.
-template <int KEY_BYTES, int VALUE_BYTES> struct SortTile {
-  static constexpr int kSubTiles = kSortBlock / kSubLanes;
+template <int KEY_BYTES, int VALUE_BYTES, int BLOCK> struct SortTile {
+  static constexpr int kSubTiles = BLOCK / kSubLanes;
   static constexpr int kCounterWords = kSubTiles * kRadix;
   static constexpr int kCounterBytes = kCounterWords * 4;
   static constexpr int kItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
-  static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES);
+  static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES, BLOCK);
   static constexpr int kSubTileKeys = kSubLanes * kItems;
   static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
   static constexpr int kStageBytes =
@@ -359,8 +370,15 @@ __device__ __forceinline__ void load_tile_keys(
 #define ILGPU_HIP_SORT_WAVES_PER_EU 4
 #endif
 
+// Tile of a group's k-th draw: its chunks are g, g + 8, g + 16, ... of
+// 2^chunk_shift consecutive tiles.
+__device__ __forceinline__ int ticket_tile(uint32_t k, uint32_t g, int chunk_shift) {
+  const uint32_t chunk = (k >> chunk_shift) * kTicketGroups + g;
+  return (int)((chunk << chunk_shift) + (k & ((1u << chunk_shift) - 1u)));
+}
+
 // Sorts one tile by the digit of `pass` and scatters it.
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT>
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT, int BLOCK>
 __device__ __forceinline__ void sort_tile(
     typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys,
@@ -373,7 +391,7 @@ __device__ __forceinline__ void sort_tile(
     const uint32_t (&hot)[kMaxHot], uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
   constexpr int kItems = TileCfg::kItems;
   constexpr int kSubTiles = TileCfg::kSubTiles;
   constexpr bool kPairs = VALUE_BYTES > 0;
@@ -400,6 +418,7 @@ __device__ __forceinline__ void sort_tile(
   const int sub = wave;                     // sub-tile index in the block
   const int first_local = sub * TileCfg::kSubTileKeys + lane;
   const int shift = pass * 8;
+
 
   auto digit = [&](K k) -> uint32_t {
     if constexpr (FLOAT_KEYS) return digit_of(k, xf, shift);
@@ -634,7 +653,7 @@ __device__ __forceinline__ void sort_tile(
   asm volatile("" : "+v"(tid));
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
-    const int i = j * kSortBlock + tid;
+    const int i = j * BLOCK + tid;
     if (FULL || i < valid) {
       const K k = s_keys[i];
       const uint32_t g = s_global_off[digit(k)] + (uint32_t)i;
@@ -658,7 +677,7 @@ __device__ __forceinline__ void sort_tile(
       __syncthreads();
 #pragma unroll
       for (int j = 0; j < kItems; ++j) {
-        const uint32_t i = (uint32_t)(j * kSortBlock + tid);
+        const uint32_t i = (uint32_t)(j * BLOCK + tid);
         if ((FULL || i < (uint32_t)valid) && i - lo < (uint32_t)kValuesPerRound)
           dst_vals[gpos[j]] = s_vals[i - lo];
       }
@@ -666,8 +685,8 @@ __device__ __forceinline__ void sort_tile(
   }
 }
 
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS>
-__global__ __launch_bounds__(kSortBlock, ILGPU_HIP_SORT_WAVES_PER_EU)
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, int BLOCK>
+__global__ __launch_bounds__(BLOCK, ILGPU_HIP_SORT_WAVES_PER_EU)
 void onesweep_kernel(
     typename KeyOf<KEY_BYTES>::type* keys_a,
     typename KeyOf<KEY_BYTES>::type* keys_b,
@@ -678,7 +697,7 @@ void onesweep_kernel(
     int values_from_index, int chunk_shift, uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES>;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
   constexpr int kTile = TileCfg::kTile;
   constexpr int kItems = TileCfg::kItems;
 
@@ -717,14 +736,13 @@ void onesweep_kernel(
   // A block draws its next tile only when it is about to start it: the time
   // between a tile's ticket and the publication of its digit counts is what
   // every later tile's look-back waits for.  (Drawing it earlier, to load the
-  // next keys during the write-out, measured 3 to 12 % slower.)  The key loads
+  // next keys during the look-back and the write-out, measured 3 to 12 % slower,
+  // with the global ticket and again with the per-group ones.)  The key loads
   // fly while the ranking counters are cleared.
   while (true) {
     if (tid == 0) {
       const uint32_t g = blockIdx.x % (uint32_t)kTicketGroups;
-      const uint32_t k = atomicAdd(ticket + g * kTicketStride, 1u);
-      const uint32_t chunk = (k >> chunk_shift) * kTicketGroups + g;
-      s_tile = (int)((chunk << chunk_shift) + (k & ((1u << chunk_shift) - 1u)));
+      s_tile = ticket_tile(atomicAdd(ticket + g * kTicketStride, 1u), g, chunk_shift);
     }
     __syncthreads();  // also: the previous tile's staged keys have been read
     const int tile = s_tile;
@@ -744,11 +762,11 @@ void onesweep_kernel(
       load_tile_keys<KEY_BYTES, kItems, kFull>(src_keys, tile_base, valid, first_local, key);
       {  // clear the ranking counters
         uint4* z = reinterpret_cast<uint4*>(s_stage);
-        for (int i = tid; i < TileCfg::kCounterBytes / 16; i += kSortBlock)
+        for (int i = tid; i < TileCfg::kCounterBytes / 16; i += BLOCK)
           z[i] = make_uint4(0u, 0u, 0u, 0u);
       }
       __syncthreads();
-      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot>(
+      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot, BLOCK>(
           key, src_keys, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl,
           status, make_index, s_stage, s_global_off, s_scan, hot, spin_limit);
     };
@@ -770,7 +788,6 @@ __global__ __launch_bounds__(kSortBlock) void lds_atomic_order_kernel(
   const int tid = threadIdx.x;
   for (int i = tid; i < (kSortBlock / kWaveSize) * kRadix; i += kSortBlock) s_counter[i] = 0u;
   __syncthreads();
-  const int lane = tid & (kWaveSize - 1);
   uint32_t* mine = s_counter + (tid / kWaveSize) * kRadix;
   unsigned long long wrong = 0;
   for (int r = 0; r < rows; ++r) {
@@ -824,6 +841,7 @@ __global__ __launch_bounds__(256) void finish_kernel(
 
 // ---- host side -------------------------------------------------------------
 std::atomic<uint32_t> g_spin_limit{kDefaultSpinLimit};
+std::atomic<int32_t> g_large_min_tiles_per_cu{-1};  // negative: the defaults above
 
 struct TempLayout {
   int64_t alt_keys, alt_vals, excl, plan, zero_begin, hist, tickets, status,
@@ -831,9 +849,11 @@ struct TempLayout {
   int64_t tiles;
 };
 
-TempLayout make_layout(int64_t n, int key_bytes, int value_bytes) {
+// Layout for tiles of `block` threads.  Temp views are sized for the small
+// block (more tiles, more status words); the large block's layout fits inside.
+TempLayout make_layout(int64_t n, int key_bytes, int value_bytes, int block = kSortBlock) {
   TempLayout L;
-  const int64_t tile = tile_keys(key_bytes, value_bytes);
+  const int64_t tile = tile_keys(key_bytes, value_bytes, block);
   L.tiles = div_up(n, tile);
   int64_t off = 0;
   L.alt_keys = off; off += align_up(n * key_bytes, 256);
@@ -877,11 +897,76 @@ KeyXform make_xform(int32_t key_type, int32_t flags) {
   return xf;
 }
 
+// The passes of one sort with tiles of BLOCK threads.
+template <int KEY_BYTES, int VALUE_BYTES, int BLOCK>
+int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L, char* base,
+                      const KeyXform& xf, int cus) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  using Val = typename ValueOf<VALUE_BYTES>::type;
+  K* keys_a = static_cast<K*>(a.keys);
+  K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
+  Val* vals_a = static_cast<Val*>(a.values);
+  Val* vals_b = reinterpret_cast<Val*>(base + L.alt_vals);
+  uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
+  SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
+  uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
+  const int passes = KEY_BYTES;
+  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
+  const bool float_keys = xf.mode != kModePlain;
+  auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false, BLOCK>;
+  if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
+    if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true, BLOCK>;
+  }
+  // Resident blocks per CU of this instantiation: asked once per device and
+  // kernel (the query costs microseconds, which small sorts would feel).
+  static std::atomic<int> cached_per_cu[kMaxCachedDevices][2];  // per instantiation
+  const int device = current_device();
+  std::atomic<int>* cached =
+      device >= 0 && device < kMaxCachedDevices ? &cached_per_cu[device][float_keys ? 1 : 0]
+                                                : nullptr;
+  int per_cu = cached ? cached->load(std::memory_order_relaxed) : 0;
+  if (per_cu == 0) {
+    ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+        &per_cu, pass_kernel, BLOCK, 0));
+    if (per_cu < 1) per_cu = 1;
+    if (cached) cached->store(per_cu, std::memory_order_relaxed);
+  }
+  int64_t grid = (int64_t)cus * per_cu;
+  if (grid > L.tiles) grid = L.tiles;
+  // Chunks as long as leave every block of the grid a tile of its own in the
+  // first round (short inputs: single tiles, handed out round-robin).
+  int chunk_shift = 0;
+  while (chunk_shift < kMaxChunkShift && (grid << (chunk_shift + 1)) <= L.tiles) ++chunk_shift;
+  const uint32_t spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+  for (int p = 0; p < passes; ++p) {
+    uint32_t* status =
+        reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
+    {
+      ProfileScope scope(stream, "sort_onesweep");
+      hipLaunchKernelGGL(pass_kernel,
+                         dim3((unsigned)grid), dim3(BLOCK), 0, stream,
+                         keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
+                         status, tickets + p * kTicketGroups * kTicketStride, plan, (int)L.tiles,
+                         from_index, chunk_shift, spin_limit);
+    }
+    ILGPU_HIP_CHECK(hipGetLastError());
+  }
+  return ILGPU_HIP_SUCCESS;
+}
+
 template <int KEY_BYTES, int VALUE_BYTES>
 int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  const TempLayout L = make_layout(a.n, KEY_BYTES, VALUE_BYTES);
+  const int cus = device_cu_count();
+  int64_t min_tiles_per_cu = g_large_min_tiles_per_cu.load(std::memory_order_relaxed);
+  if (min_tiles_per_cu < 0)
+    min_tiles_per_cu = VALUE_BYTES > 0 ? kLargeMinTilesPerCuPairs : kLargeMinTilesPerCuKeys;
+  const bool use_large =
+      div_up(a.n, (int64_t)tile_keys(KEY_BYTES, VALUE_BYTES, kSortBlockLarge)) >=
+      min_tiles_per_cu * cus;
+  const TempLayout L =
+      make_layout(a.n, KEY_BYTES, VALUE_BYTES, use_large ? kSortBlockLarge : kSortBlock);
   char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)a.temp, 256));
   K* keys_a = static_cast<K*>(a.keys);
   K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
@@ -890,10 +975,8 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
   SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
   uint32_t* hist = reinterpret_cast<uint32_t*>(base + L.hist);
-  uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
   const KeyXform xf = make_xform(a.key_type, a.flags);
   const int passes = KEY_BYTES;
-  const int cus = device_cu_count();
   const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
 
   int32_t rc = launch_zero_words(stream, hist, (L.total - L.zero_begin) / 4);
@@ -922,45 +1005,11 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   }
   ILGPU_HIP_CHECK(hipGetLastError());
 
-  const bool float_keys = xf.mode != kModePlain;
-  auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false>;
-  if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
-    if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true>;
-  }
-  // Resident blocks per CU of this instantiation: asked once per device and
-  // kernel (the query costs microseconds, which small sorts would feel).
-  static std::atomic<int> cached_per_cu[kMaxCachedDevices][2];
-  const int device = current_device();
-  std::atomic<int>* cached =
-      device >= 0 && device < kMaxCachedDevices ? &cached_per_cu[device][float_keys ? 1 : 0]
-                                                : nullptr;
-  int per_cu = cached ? cached->load(std::memory_order_relaxed) : 0;
-  if (per_cu == 0) {
-    ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
-        &per_cu, pass_kernel, kSortBlock, 0));
-    if (per_cu < 1) per_cu = 1;
-    if (cached) cached->store(per_cu, std::memory_order_relaxed);
-  }
-  int64_t grid = (int64_t)cus * per_cu;
-  if (grid > L.tiles) grid = L.tiles;
-  // Chunks as long as leave every block of the grid a tile of its own in the
-  // first round (short inputs: single tiles, handed out round-robin).
-  int chunk_shift = 0;
-  while (chunk_shift < kMaxChunkShift && (grid << (chunk_shift + 1)) <= L.tiles) ++chunk_shift;
-  const uint32_t spin_limit = g_spin_limit.load(std::memory_order_relaxed);
-  for (int p = 0; p < passes; ++p) {
-    uint32_t* status =
-        reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
-    {
-      ProfileScope scope(stream, "sort_onesweep");
-      hipLaunchKernelGGL(pass_kernel,
-                         dim3((unsigned)grid), dim3(kSortBlock), 0, stream,
-                         keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
-                         status, tickets + p * kTicketGroups * kTicketStride, plan, (int)L.tiles,
-                         from_index, chunk_shift, spin_limit);
-    }
-    ILGPU_HIP_CHECK(hipGetLastError());
-  }
+  if (use_large)
+    rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlockLarge>(stream, a, L, base, xf, cus);
+  else
+    rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlock>(stream, a, L, base, xf, cus);
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
   {
     int64_t blocks = div_up(a.n, 256);
     if (blocks > (int64_t)cus * 8) blocks = (int64_t)cus * 8;
@@ -1049,8 +1098,11 @@ int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
 
 }  // namespace
 
-void set_sort_lookback_spin_limit(int32_t polls) {
-  g_spin_limit.store(polls < 0 ? kDefaultSpinLimit : (uint32_t)polls, std::memory_order_relaxed);
+void set_sort_parameter(int32_t parameter, int32_t value) {
+  if (parameter == ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT)
+    g_spin_limit.store(value < 0 ? kDefaultSpinLimit : (uint32_t)value, std::memory_order_relaxed);
+  else
+    g_large_min_tiles_per_cu.store(value < 0 ? -1 : value, std::memory_order_relaxed);
 }
 
 int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches) {

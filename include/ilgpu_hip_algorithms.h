@@ -189,17 +189,28 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void *keys,
 int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
                                             int32_t rows, int64_t *mismatches);
 
-/* How long the look-back of a sort pass polls the status word of an earlier
- * tile that has published nothing before it stops waiting and counts that
- * tile's digit itself from the source keys (the sort's tiles are handed to
- * fixed groups of blocks, so a tile may wait for one whose group has no
- * resident block; with this bound every block finishes whatever the others
- * do).  polls < 0 restores the default (4096); 0 makes every look-back that
- * meets an empty word take the slow path at once, which is how the tests
- * exercise it.  Process-wide, applies to sorts launched afterwards.  No
- * counterpart in the reference (its passes are separate kernel launches,
- * RadixSortExtensions.cs:1276-1334). */
-int32_t ilgpu_hip_set_sort_lookback_spin_limit(int32_t polls);
+/* Two process-wide parameters of the sort, for tests and tuning; they apply to
+ * sorts launched afterwards, a negative value restores the default, and neither
+ * has a counterpart in the reference (its passes are separate kernel launches,
+ * RadixSortExtensions.cs:1276-1334).
+ *   LOOKBACK_SPIN_LIMIT  how often the look-back of a pass polls the status
+ *     word of an earlier tile that has published nothing before it stops
+ *     waiting and counts that tile's digit itself from the source keys (tiles
+ *     are handed to fixed groups of blocks, so a tile may wait for one whose
+ *     group has no resident block; with this bound every block finishes
+ *     whatever the others do).  Default 4096; 0 makes every look-back that
+ *     meets an empty word take the slow path at once, which is how the tests
+ *     exercise it.
+ *   LARGE_BLOCK_MIN_TILES_PER_CU  inputs of at least this many 1024-thread
+ *     tiles per compute unit are sorted with 1024-thread blocks (longer runs
+ *     per digit), smaller ones with 512-thread blocks (more blocks for fewer
+ *     keys).  Default 10 for keys, 2 for pairs; 0 = always the large block,
+ *     INT32_MAX = never. */
+enum {
+  ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0,
+  ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1
+};
+int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value);
 
 /* ---- scan ---------------------------------------------------------------
  * Replaces: Scan<T,TStrideIn,TStrideOut> delegates made by CreateScan(kind)

@@ -622,7 +622,7 @@ def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
     # look-back can meet a predecessor nobody has started; past a bound of polls
     # it counts that tile's digit itself from the source keys.  With the bound
     # at zero every empty status word takes that path; results must not change.
-    capi.set_sort_lookback_spin_limit(0)
+    capi.sort_set_parameter(capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT, 0)
     try:
         for dtype, n in [(np.uint32, 18432 * 40 + 77), (np.uint8, 300000), (np.int16, 400001),
                          (np.uint64, 9216 * 33 + 5)]:
@@ -642,11 +642,78 @@ def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
         k, v = gpu_sort_pairs(keys, values)
         order = np.argsort(keys, kind="stable")
         assert np.array_equal(k, keys[order]) and np.array_equal(v, values[order])
+        # the same with 1024-thread blocks
+        capi.sort_set_parameter(capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU, 0)
+        keys = random_ints(np.uint32, 36864 * 20 + 77, seed=17)
+        assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+        keys = random_ints(np.uint16, 300000, seed=18, lo=0, hi=99)
+        values = np.arange(keys.size, dtype=np.uint32)
+        k, v = gpu_sort_pairs(keys, values)
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(k, keys[order]) and np.array_equal(v, values[order])
     finally:
-        capi.set_sort_lookback_spin_limit(-1)
-    # back on the default bound
+        capi.sort_set_parameter(capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT, -1)
+        capi.sort_set_parameter(capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU, -1)
+    # back on the defaults
     keys = random_ints(np.uint32, 18432 * 40 + 77, seed=16)
     assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+    with pytest.raises(capi.ArgumentOutOfRangeError):
+        capi.sort_set_parameter(7, 0)
+
+
+@pytest.fixture
+def large_sort_blocks():
+    """Sorts of any size take the 1024-thread kernels (by default only inputs of
+    tens of millions of keys do)."""
+    capi.sort_set_parameter(capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU, 0)
+    yield
+    capi.sort_set_parameter(capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU, -1)
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_with_large_blocks_matches_oracle(large_sort_blocks, dtype, descending):
+    kinds = np.dtype(dtype).kind
+    for n in [1, 65, 36863, 36864, 36865, 100003]:
+        note("large-block sort", np.dtype(dtype).name, descending, n)
+        keys = random_float_bits(dtype, n, seed=n) if kinds == "f" else random_ints(dtype, n, seed=n)
+        assert bits_equal(gpu_sort(keys, descending=descending),
+                          O.radix_sort(keys, descending=descending)), n
+
+
+@pytest.mark.parametrize("key_dtype,value_dtype", [
+    (np.uint32, np.uint32), (np.uint64, np.uint32), (np.uint32, np.uint64), (np.int64, np.float64),
+    (np.uint8, np.uint8), (np.int16, np.uint16), (np.float32, np.int32), (np.float16, np.uint64)])
+def test_sort_pairs_with_large_blocks_are_stable(large_sort_blocks, key_dtype, value_dtype):
+    for n in [1000, 8191 * 2 + 5, 120001]:
+        note("large-block pairs", np.dtype(key_dtype).name, np.dtype(value_dtype).name, n)
+        # few distinct keys: stability decides the value order
+        keys = (random_ints(np.int32, n, seed=n, lo=-40, hi=40)).astype(key_dtype)
+        values = np.arange(n).astype(value_dtype)
+        k, v = gpu_sort_pairs(keys, values)
+        ek, ev = O.radix_sort_pairs(keys, values)
+        assert bits_equal(k, ek) and bits_equal(v, ev), n
+    # 16-byte values and index-generated values
+    n = 50000
+    keys = random_ints(np.uint32, n, seed=5, lo=0, hi=300)
+    order = np.argsort(keys, kind="stable")
+    values = np.zeros((n, 2), dtype=np.uint64)
+    values[:, 0] = np.arange(n)
+    values[:, 1] = ~np.arange(n, dtype=np.uint64)
+    dk = D.from_numpy(keys)
+    dv = D(n, np.dtype([("a", np.uint64), ("b", np.uint64)]),
+           _bytes=D.from_numpy(values.reshape(-1)).bytes)
+    temp = capi.temp_buffer(capi.radix_sort_temp_bytes(n, np.uint32, 16))
+    capi.check(capi.lib().ilgpu_hip_radix_sort_pairs(
+        None, dk.ptr, 1, dv.ptr, 1, n, capi.U32, 16, 0, capi.VALUES_FROM_VIEW,
+        temp.ptr, temp.nbytes))
+    sync()
+    assert np.array_equal(dk.numpy(), keys[order])
+    assert np.array_equal(dv.bytes.cpu().numpy().view(np.uint64).reshape(n, 2), values[order])
+    dk2, dv2 = D.from_numpy(keys), D.zeros(n, np.uint32)
+    capi.radix_sort_pairs(dk2, dv2, values_from_index=True)
+    sync()
+    assert np.array_equal(dk2.numpy(), keys[order]) and np.array_equal(dv2.numpy(), order)
 
 
 @pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
