@@ -1244,6 +1244,39 @@ def test_two_streams_run_independent_calls_concurrently():
         assert d_sum[i].numpy()[0] == O.reduce(vals), i
 
 
+def test_two_sorts_on_two_streams_share_the_gpu():
+    # Each sort's pass kernels are persistent and sized to fill the GPU, so two
+    # of them on two streams can each hold only part of the compute units.  A
+    # pass hands its tiles to fixed groups of blocks; no block may wait without
+    # bound for a tile whose group is not resident (the look-back gives up on an
+    # unpublished tile and counts it itself), so both sorts finish and are exact.
+    import torch
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    n1, n2 = (1 << 24) + 11, (1 << 24) - 5
+    a = datagen.uniform_u32(n1)
+    b = datagen.uniform_u64(n2)
+    d_a = [D.from_numpy(a) for _ in range(3)]
+    d_b = [D.from_numpy(b) for _ in range(3)]
+    d_v = [D.zeros(n2, np.uint32) for _ in range(3)]
+    t_a = [capi.temp_buffer(capi.radix_sort_temp_bytes(n1, np.uint32)) for _ in range(3)]
+    t_b = [capi.temp_buffer(capi.radix_sort_temp_bytes(n2, np.uint64, 4)) for _ in range(3)]
+    torch.cuda.synchronize()
+    note("two sorts on two streams", n1, n2)
+    for i in range(3):
+        with torch.cuda.stream(s1):
+            capi.radix_sort_keys(d_a[i], t_a[i])
+        with torch.cuda.stream(s2):
+            capi.radix_sort_pairs(d_b[i], d_v[i], t_b[i], values_from_index=True)
+    s1.synchronize()
+    s2.synchronize()
+    e_a = np.sort(a, kind="stable")
+    order = np.argsort(b, kind="stable")
+    for i in range(3):
+        assert np.array_equal(d_a[i].numpy(), e_a), i
+        assert np.array_equal(d_b[i].numpy(), b[order]), i
+        assert np.array_equal(d_v[i].numpy(), order.astype(np.uint32)), i
+
+
 def test_calls_can_be_captured_into_a_graph_and_replayed():
     # Every call is stream-ordered kernels only (temp memory is cleared by a
     # fill kernel, nothing is allocated), so a sequence of calls can be
