@@ -28,7 +28,8 @@
 // Key order: digit(k) = ((k ^ xor_mask ^ f(k)) >> shift) & 0xFF, where
 // xor_mask folds the sign-bit flip of signed/float types and the complement
 // of Descending* (RadixSortOperations.tt:77-93, 122-123) and f(k) is the
-// per-key term of the float transforms.
+// per-key term of the float transforms.  Float keys are converted once, by the
+// first pass that runs, and converted back by the last one.
 //
 // Algorithmic HBM traffic for n keys of k bytes, values of v bytes and P
 // executed passes: n * (k * (2P + 1) + v * 2P) bytes.
@@ -160,30 +161,43 @@ constexpr int tile_keys(int key_bytes, int value_bytes, int block) {
 }
 
 // How raw key bits map to unsigned bits that sort in the requested order.
-enum { kModePlain = 0, kModeFloatReference = 1, kModeFloatTotalOrder = 2 };
+// ordered(k) = k ^ xor_mask ^ (lsr(~k, bits-1) & reference_term) ^ (asr(k, bits-1) & total_term):
+// branch-free for every mode.  reference_term is 1 for the float order of the
+// reference (RadixSortOperations.tt:81-89 as written: the complement mask is a
+// LOGICAL shift of ~bits, i.e. 1 for non-negative values and 0 otherwise);
+// total_term is all bits below the sign for IEEE totalOrder (negative values
+// have them flipped); both are 0 for integer keys.
 struct KeyXform {
   uint64_t xor_mask;
-  int32_t mode;
+  uint64_t reference_term;
+  uint64_t total_term;
 };
 
 template <typename K>
-__device__ __forceinline__ K ordered_bits(K k, const KeyXform& xf) {
+__device__ __forceinline__ K key_term(K k, const KeyXform& xf) {
   constexpr int kBits = sizeof(K) * 8;
-  K o = k ^ (K)xf.xor_mask;
-  if (xf.mode == kModeFloatReference) {
-    // RadixSortOperations.tt:81-89 as written: the complement mask is a
-    // LOGICAL shift of ~bits, i.e. 1 for non-negative values and 0 otherwise.
-    o ^= (K)((K)(~k) >> (kBits - 1));
-  } else if (xf.mode == kModeFloatTotalOrder) {
-    const K sign = (K)((K)1 << (kBits - 1));
-    if (k & sign) o ^= (K)(sign - 1);
-  }
-  return o;
+  using S = typename std::make_signed<K>::type;
+  return (K)(((K)((K)(~k) >> (kBits - 1)) & (K)xf.reference_term) ^
+             ((K)((S)k >> (kBits - 1)) & (K)xf.total_term));
+}
+
+template <typename K>
+__device__ __forceinline__ K ordered_bits(K k, const KeyXform& xf) {
+  return (K)(k ^ (K)xf.xor_mask ^ key_term(k, xf));
 }
 
 template <typename K>
 __device__ __forceinline__ uint32_t digit_of(K k, const KeyXform& xf, int shift) {
   return (uint32_t)(ordered_bits(k, xf) >> shift) & (kRadix - 1);
+}
+
+// Inverse of ordered_bits.  The per-key term depends on the key's sign bit
+// only and never changes it, so u = o ^ xor_mask has the sign bit of the key
+// and the same term taken from u gives the key back.
+template <typename K>
+__device__ __forceinline__ K raw_bits(K o, const KeyXform& xf) {
+  const K u = (K)(o ^ (K)xf.xor_mask);
+  return (K)(u ^ key_term(u, xf));
 }
 
 constexpr uint32_t kNoHotDigit = 0xFFFFFFFFu;
@@ -196,6 +210,7 @@ struct SortPlan {
   // frequent first; unused entries are kNoHotDigit.
   uint32_t hot[kMaxPasses][kMaxHot];
   uint32_t first_executed;          // index of the first pass that runs
+  uint32_t last_executed;           // index of the last pass that runs
   uint32_t executed;                // number of passes that run
   uint32_t final_in_alt;            // result sits in the alternate buffer
 };
@@ -213,8 +228,10 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
   __syncthreads();
 
   const uint32_t replica = threadIdx.x & ((1u << replica_shift) - 1u);
+  const bool has_term = (xf.reference_term | xf.total_term) != 0;  // float keys
   auto count = [&](K k) {
-    const K o = ordered_bits(k, xf);
+    K o = (K)(k ^ (K)xf.xor_mask);
+    if (has_term) o ^= key_term(k, xf);
 #pragma unroll
     for (int p = 0; p < (int)sizeof(K); ++p) {
       const uint32_t d = (uint32_t)(o >> (8 * p)) & (kRadix - 1);
@@ -273,7 +290,7 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
   const int d = threadIdx.x;
   const int lane = d & (kWaveSize - 1);
   const int wave = d / kWaveSize;
-  uint32_t parity = 0, executed = 0, first = passes;
+  uint32_t parity = 0, executed = 0, first = passes, last = passes;
   for (int p = 0; p < passes; ++p) {
     if (d < kMaxHot) s_hot[d] = 0ull;
     if (d == 0) s_trivial = 0;
@@ -309,6 +326,7 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
     }
     if (!trivial) {
       if (executed == 0) first = p;
+      last = p;
       parity ^= 1u;
       ++executed;
     }
@@ -316,6 +334,7 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
   }
   if (d == 0) {
     plan->first_executed = first;
+    plan->last_executed = last;
     plan->executed = executed;
     plan->final_in_alt = parity;
   }
@@ -388,7 +407,7 @@ __device__ __forceinline__ void sort_tile(
     int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
     const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
     unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan,
-    const uint32_t (&hot)[kMaxHot], uint32_t spin_limit) {
+    const uint32_t (&hot)[kMaxHot], uint32_t spin_limit, bool in_raw, bool out_raw) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
@@ -420,8 +439,15 @@ __device__ __forceinline__ void sort_tile(
   const int shift = pass * 8;
 
 
+  // Float keys travel between the passes in their ordered form: the first
+  // pass that runs converts them as it ranks them (in_raw), the last one
+  // converts them back as it writes them (out_raw), and in between a digit is
+  // a shift and a mask.  Other keys keep their bits; their order is one xor.
+  // (A pass that finds them converted applies the identity: no mask, no term.)
+  KeyXform xf_in = xf;
+  if (!in_raw) xf_in = KeyXform{0, 0, 0};
   auto digit = [&](K k) -> uint32_t {
-    if constexpr (FLOAT_KEYS) return digit_of(k, xf, shift);
+    if constexpr (FLOAT_KEYS) return (uint32_t)(k >> shift) & (kRadix - 1);
     else return (uint32_t)((K)(k ^ (K)xf.xor_mask) >> shift) & (kRadix - 1);
   };
   // Keys past the end of the input take digit 255; they come last in memory
@@ -630,7 +656,11 @@ __device__ __forceinline__ void sort_tile(
             const K* other = src_keys + (int64_t)(t - u) * TileCfg::kTile;
             uint32_t c = 0;
 #pragma unroll 4
-            for (int i = 0; i < TileCfg::kTile; ++i) c += digit(other[i]) == (uint32_t)tid;
+            for (int i = 0; i < TileCfg::kTile; ++i) {
+              K k = other[i];
+              if constexpr (FLOAT_KEYS) k = ordered_bits(k, xf_in);
+              c += digit(k) == (uint32_t)tid;
+            }
             s[u] = status_aggregate(c);
             break;
           }
@@ -657,7 +687,8 @@ __device__ __forceinline__ void sort_tile(
     if (FULL || i < valid) {
       const K k = s_keys[i];
       const uint32_t g = s_global_off[digit(k)] + (uint32_t)i;
-      dst_keys[g] = k;
+      if constexpr (FLOAT_KEYS) dst_keys[g] = out_raw ? raw_bits(k, xf) : k;
+      else dst_keys[g] = k;
       if constexpr (kPairs) gpos[j] = g;
     }
     constexpr int kWriteGroup = kPairs ? ILGPU_HIP_SORT_PAIR_WRITE_GROUP : ILGPU_HIP_SORT_WRITE_GROUP;
@@ -717,6 +748,8 @@ void onesweep_kernel(
   Val* dst_vals = src_alt ? vals_a : vals_b;
   const bool make_index = VALUE_BYTES > 0 && values_from_index &&
                           plan->first_executed == (uint32_t)pass;
+  const bool in_raw = plan->first_executed == (uint32_t)pass;
+  const bool out_raw = plan->last_executed == (uint32_t)pass;
   const int tid = threadIdx.x;
   const int first_local = (tid / kSubLanes) * TileCfg::kSubTileKeys + tid % kSubLanes;
 
@@ -760,6 +793,12 @@ void onesweep_kernel(
       constexpr bool kHot = decltype(with_hot)::value;
       K key[kItems];
       load_tile_keys<KEY_BYTES, kItems, kFull>(src_keys, tile_base, valid, first_local, key);
+      if constexpr (FLOAT_KEYS) {
+        if (in_raw) {
+#pragma unroll
+          for (int j = 0; j < kItems; ++j) key[j] = ordered_bits(key[j], xf);
+        }
+      }
       {  // clear the ranking counters
         uint4* z = reinterpret_cast<uint4*>(s_stage);
         for (int i = tid; i < TileCfg::kCounterBytes / 16; i += BLOCK)
@@ -768,7 +807,7 @@ void onesweep_kernel(
       __syncthreads();
       sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot, BLOCK>(
           key, src_keys, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl,
-          status, make_index, s_stage, s_global_off, s_scan, hot, spin_limit);
+          status, make_index, s_stage, s_global_off, s_scan, hot, spin_limit, in_raw, out_raw);
     };
     if (valid != kTile) run(std::false_type{}, std::true_type{});
     else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
@@ -874,7 +913,7 @@ KeyXform make_xform(int32_t key_type, int32_t flags) {
   const int bits = elem_size(key_type) * 8;
   const uint64_t all = bits == 64 ? ~0ull : ((1ull << bits) - 1ull);
   const uint64_t sign = 1ull << (bits - 1);
-  KeyXform xf{0, kModePlain};
+  KeyXform xf{0, 0, 0};
   switch (key_type) {
     case ILGPU_HIP_I8: case ILGPU_HIP_I16: case ILGPU_HIP_I32: case ILGPU_HIP_I64:
       xf.xor_mask = sign;
@@ -882,12 +921,12 @@ KeyXform make_xform(int32_t key_type, int32_t flags) {
     case ILGPU_HIP_F16: case ILGPU_HIP_F32: case ILGPU_HIP_F64:
       if (flags & ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER) {
         xf.xor_mask = sign;
-        xf.mode = kModeFloatTotalOrder;
+        xf.total_term = sign - 1ull;
       } else {
         // Half: (uint)~bits >> 15 keeps the sign-extended upper ones, so bits
         // 1..15 are always flipped (RadixSortOperations.tt:77-80).
         xf.xor_mask = key_type == ILGPU_HIP_F16 ? 0xFFFEull : sign;
-        xf.mode = kModeFloatReference;
+        xf.reference_term = 1ull;
       }
       break;
     default:
@@ -912,7 +951,7 @@ int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L
   uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
   const int passes = KEY_BYTES;
   const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
-  const bool float_keys = xf.mode != kModePlain;
+  const bool float_keys = (xf.reference_term | xf.total_term) != 0;
   auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false, BLOCK>;
   if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
     if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true, BLOCK>;

@@ -362,6 +362,38 @@ def test_sort_float_types_match_reference_order(dtype, descending):
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_float_keys_when_passes_are_skipped(dtype, descending):
+    # Float keys are converted to their ordered form by the first pass that runs
+    # and back by the last one; passes whose digit is the same for every key do
+    # not run at all.  Inputs that skip the top pass (one exponent), the bottom
+    # passes (few mantissa bits), everything but one pass, and every pass.
+    rng = np.random.default_rng(7)
+    n = 70001
+    one_exponent = (1.0 + rng.random(n)).astype(dtype)              # [1, 2): top digit constant
+    coarse = (rng.integers(-8, 8, n) * 0.5).astype(dtype)           # low mantissa bytes all zero
+    one_pass = np.where(rng.random(n) < 0.5, 1.0, 1.5).astype(dtype)
+    constant = np.full(n, -2.5, dtype=dtype)
+    for name, keys in [("one exponent", one_exponent), ("coarse", coarse),
+                       ("two values", one_pass), ("constant", constant)]:
+        note("float keys with skipped passes", np.dtype(dtype).name, descending, name)
+        expect = O.radix_sort(keys, descending=descending)
+        assert bits_equal(gpu_sort(keys, descending=descending), expect), name
+        values = np.arange(n, dtype=np.uint32)
+        ek, ev = O.radix_sort_pairs(keys, values, descending=descending)
+        k, v = gpu_sort_pairs(keys, values, descending=descending)
+        assert bits_equal(k, ek) and np.array_equal(v, ev), name
+    u = {2: np.uint16, 4: np.uint32, 8: np.uint64}[np.dtype(dtype).itemsize]
+    bits = coarse.view(u)
+    sign = u(1) << u(np.dtype(dtype).itemsize * 8 - 1)
+    ordered = np.where(bits & sign, ~bits, bits | sign)
+    if descending:
+        ordered = ~ordered
+    expect = coarse[np.argsort(ordered, kind="stable")]
+    assert bits_equal(gpu_sort(coarse, descending=descending, float_total_order=True), expect)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
 def test_sort_float_total_order_flag(dtype):
     # Extension without a reference counterpart: IEEE totalOrder.
     keys = random_float_bits(dtype, 20000, seed=4)
