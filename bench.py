@@ -92,9 +92,16 @@ CSRC = os.path.join(ROOT, "ilgpu_amd", "csrc")
 
 
 def source_digest(file_name):
+    """Digest of a kernel source's code: // comments, indentation and blank
+    lines do not count, so that only a change of code makes the counters stale."""
     import hashlib
-    with open(os.path.join(CSRC, file_name), "rb") as f:
-        return hashlib.sha256(f.read()).hexdigest()[:16]
+    lines = []
+    with open(os.path.join(CSRC, file_name), encoding="utf-8") as f:
+        for line in f:
+            code = line.split("//", 1)[0].strip()
+            if code:
+                lines.append(code)
+    return hashlib.sha256("\n".join(lines).encode()).hexdigest()[:16]
 
 
 def measured_traffic(workload, default_size):

@@ -381,10 +381,11 @@ __device__ __forceinline__ void load_tile_keys(
   }
 }
 
-// Waves per SIMD the pass kernel is compiled for: two blocks of eight waves
-// per CU.  That bounds a thread at 128 registers (36 keys and 18 registers of
-// packed ranks in a keys-only sort; fewer items when values ride along) and a
-// block at 80 KiB of LDS (the 36-key tile stages 72 KiB).
+// Waves per SIMD the pass kernel is compiled for: sixteen waves per CU, as two
+// 512-thread blocks or one 1024-thread block.  That bounds a thread at 128
+// registers (36 keys and 18 registers of packed ranks in a keys-only sort;
+// fewer items when values ride along) and the blocks of a CU at 160 KiB of
+// LDS together (a 36-key tile stages 72 KiB per 512 threads).
 #ifndef ILGPU_HIP_SORT_WAVES_PER_EU
 #define ILGPU_HIP_SORT_WAVES_PER_EU 4
 #endif
