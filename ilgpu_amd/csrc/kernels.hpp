@@ -32,7 +32,7 @@ int32_t launch_histogram(hipStream_t stream, const void* in, int64_t n,
                          int64_t num_bins, int32_t bin_type, int32_t locator,
                          int32_t* overflow);
 
-// radix_sort.hip
+// radix_sort.hip (kernels: radix_sort_impl.hpp, radix_sort_k*.hip)
 struct SortArgs {
   void* keys;
   void* values;      // nullptr for a keys-only sort

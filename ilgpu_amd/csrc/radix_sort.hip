@@ -1,820 +1,21 @@
-// Radix sort of keys and key/value pairs: onesweep LSD sort, 8-bit digits.
-//
-// Stands in for the RadixSort / RadixSortPairs delegates of
-// RadixSortExtensions.cs:1017-1337.  The reference runs NumBits/2 passes of
-// {memset, local 4-way split, counter scan, scatter} (:1276-1334) and packs
-// pairs into an array of structs first (:1057-1072).  Here a sort of k-byte
-// keys is
-//
-//   zero      clears the global digit histograms, tile tickets and look-back
-//             status words (one launch);
-//   histogram one read of the keys builds the 256-bin histogram of every digit
-//             position in LDS (replicated counters) and adds it to global;
-//   plan      one block turns the histograms into exclusive digit offsets,
-//             marks passes whose digit is the same for every key (they are
-//             skipped) and records which buffer each pass reads;
-//   pass x k  onesweep: a block takes a tile by ticket, ranks its keys (one
-//             returning LDS add per key on per-wave digit counters; the LDS
-//             serves the lanes of an instruction in lane order, so equal digits
-//             keep memory order: every pass is stable), publishes
-//             its 256 digit counts, resolves the counts of all earlier tiles by
-//             decoupled look-back, stages the tile in digit order through LDS
-//             and writes each digit's run to its final place;
-//   finish    copies the result back if an odd number of passes ran.
-//
-// Keys and values stay in separate arrays (structure of arrays); a value
-// travels with its key through the same tile-local permutation.
-//
-// Key order: digit(k) = ((k ^ xor_mask ^ f(k)) >> shift) & 0xFF, where
-// xor_mask folds the sign-bit flip of signed/float types and the complement
-// of Descending* (RadixSortOperations.tt:77-93, 122-123) and f(k) is the
-// per-key term of the float transforms.  Float keys are converted once, by the
-// first pass that runs, and converted back by the last one.
-//
-// Algorithmic HBM traffic for n keys of k bytes, values of v bytes and P
-// executed passes: n * (k * (2P + 1) + v * 2P) bytes.
-#include <atomic>
-#include <type_traits>
-
-#include "kernels.hpp"
+// Radix sort: what does not depend on the key size — process-wide parameters,
+// the device self-test of the LDS property the ranking rests on, strided
+// views, temp sizing and the dispatch to the translation units of the key
+// sizes (radix_sort_k1/2/4/8.hip, which instantiate radix_sort_impl.hpp).
+#include "radix_sort_impl.hpp"
 
 namespace ilgpu_hip {
 
+std::atomic<uint32_t> g_sort_spin_limit{kDefaultSpinLimit};
+std::atomic<int32_t> g_sort_large_min_tiles_per_cu{-1};
+
+// radix_sort_k<bytes>.hip
+int32_t launch_sort_key_bytes_1(hipStream_t stream, const SortArgs& a);
+int32_t launch_sort_key_bytes_2(hipStream_t stream, const SortArgs& a);
+int32_t launch_sort_key_bytes_4(hipStream_t stream, const SortArgs& a);
+int32_t launch_sort_key_bytes_8(hipStream_t stream, const SortArgs& a);
+
 namespace {
-
-constexpr int kRadix = 256;
-constexpr int kMaxPasses = 8;
-// Launch shape of the onesweep pass.  The block size fixes the number of
-// per-wave sub-tiles (and with it the LDS footprint of the ranking counters);
-// items per thread fix the tile size.
-#ifndef ILGPU_HIP_SORT_BLOCK
-#define ILGPU_HIP_SORT_BLOCK 512
-#endif
-#ifndef ILGPU_HIP_SORT_ITEMS
-#define ILGPU_HIP_SORT_ITEMS 36
-#endif
-#ifndef ILGPU_HIP_SORT_ITEMS8
-#define ILGPU_HIP_SORT_ITEMS8 18
-#endif
-#ifndef ILGPU_HIP_SORT_PAIR_ITEMS3
-#define ILGPU_HIP_SORT_PAIR_ITEMS3 16
-#endif
-#ifndef ILGPU_HIP_SORT_LOOKBACK
-#define ILGPU_HIP_SORT_LOOKBACK 4
-#endif
-// Rows whose LDS operations are in flight together while ranking, and staged
-// keys a thread reads per batch of the write-out.
-#ifndef ILGPU_HIP_SORT_RANK_GROUP
-#define ILGPU_HIP_SORT_RANK_GROUP 6
-#endif
-#ifndef ILGPU_HIP_SORT_PAIR_RANK_GROUP
-#define ILGPU_HIP_SORT_PAIR_RANK_GROUP 2
-#endif
-#ifndef ILGPU_HIP_SORT_PAIR_WRITE_GROUP
-#define ILGPU_HIP_SORT_PAIR_WRITE_GROUP 4
-#endif
-// Tiles are handed out in chunks of consecutive tiles, one chunk at a time to
-// each of kTicketGroups groups of blocks (block b is in group b % 8: blocks are
-// dispatched round-robin over the eight XCDs, so a group is the blocks of one
-// XCD).  Neighbouring tiles write neighbouring runs; when they run on one XCD
-// the partially written lines between their runs merge in that XCD's L2.
-#ifndef ILGPU_HIP_SORT_MAX_CHUNK_SHIFT
-#define ILGPU_HIP_SORT_MAX_CHUNK_SHIFT 3
-#endif
-constexpr int kTicketGroups = 8;
-constexpr int kTicketStride = 32;          // words: one 128-byte line per group
-constexpr int kMaxChunkShift = ILGPU_HIP_SORT_MAX_CHUNK_SHIFT;
-// Polls of an empty status word before a look-back stops waiting for the tile
-// and counts its digit itself.
-constexpr uint32_t kDefaultSpinLimit = 4096;
-#ifndef ILGPU_HIP_SORT_WRITE_GROUP
-#define ILGPU_HIP_SORT_WRITE_GROUP 12
-#endif
-// Two block sizes.  Large inputs take 1024-thread blocks, one per compute unit:
-// twice the tile, so every digit's run is twice as long (it is run length that
-// the scattered writes pay for, pairs above all, whose tiles are short), and
-// half as many tiles to chain.  Smaller inputs take 512-thread blocks, two per
-// compute unit, which fill the GPU with fewer keys.
-constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;      // small inputs, and the self-test
-constexpr int kSortBlockLarge = 1024;
-// The large block is used from this many of its tiles per compute unit on
-// (measured crossovers: 2^28 / 2^27 u32 keys gain 3 % / 1 %, 2^26 lose 4 %;
-// pairs of u64 keys and u32 values gain 4 to 8 % from 2^23 pairs on).
-constexpr int kLargeMinTilesPerCuKeys = 10;
-constexpr int kLargeMinTilesPerCuPairs = 2;
-// Lanes that rank together (a sub-tile row): one wave.
-constexpr int kSubLanes = kWaveSize;
-constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
-constexpr int kHistBlock = 512;
-#ifndef ILGPU_HIP_SORT_HIST_LDS_WORDS
-#define ILGPU_HIP_SORT_HIST_LDS_WORDS 16384
-#endif
-constexpr int kHistLdsWords = ILGPU_HIP_SORT_HIST_LDS_WORDS;
-// Look-back status word of a (tile, digit): 0 = nothing published yet;
-// top bits 11 = the tile's own count in the low 30 bits (a count is at most a
-// tile); anything else = inclusive count over all tiles up to this one, plus
-// one.  An inclusive count is at most n <= 2^31 - 1, so count + 1 <= 2^31
-// never has both top bits set and is never 0.
-constexpr uint32_t kStatusAggregate = 3u << 30;
-constexpr uint32_t kStatusCountMask = (1u << 30) - 1u;
-__device__ __forceinline__ uint32_t status_aggregate(uint32_t count) {
-  return kStatusAggregate | count;
-}
-__device__ __forceinline__ uint32_t status_prefix(uint32_t inclusive) { return inclusive + 1u; }
-__device__ __forceinline__ bool status_is_aggregate(uint32_t w) {
-  return (w & kStatusAggregate) == kStatusAggregate;
-}
-// Value of a non-empty word and whether it ends the look-back.
-__device__ __forceinline__ uint32_t status_value(uint32_t w) {
-  return status_is_aggregate(w) ? w & kStatusCountMask : w - 1u;
-}
-constexpr int64_t kMaxSortLength = 0x7fffffffll;  // like the reference: int.MaxValue
-
-template <int KEY_BYTES> struct KeyOf;
-template <> struct KeyOf<1> { using type = uint8_t; };
-template <> struct KeyOf<2> { using type = uint16_t; };
-template <> struct KeyOf<4> { using type = uint32_t; };
-template <> struct KeyOf<8> { using type = uint64_t; };
-
-struct alignas(16) Bytes16 { uint32_t x, y, z, w; };
-template <int VALUE_BYTES> struct ValueOf { using type = uint8_t; };
-template <> struct ValueOf<2> { using type = uint16_t; };
-template <> struct ValueOf<4> { using type = uint32_t; };
-template <> struct ValueOf<8> { using type = uint64_t; };
-template <> struct ValueOf<16> { using type = Bytes16; };
-
-// Keys per thread and tile.  Long tiles pay: the runs they scatter are longer
-// (fewer partial cache lines) and there are fewer tiles to chain.  Keys-only
-// sorts take 36 keys of up to 4 bytes or 18 of 8 bytes per thread: the most
-// that lets two blocks share a compute unit's 160 KiB of LDS.  Values live in
-// registers next to the keys, which caps pairs lower, by the registers one
-// pair takes: 20 items at two (key and value of up to 4 bytes each), 16 at
-// three, 14 at four, 8 with 16-byte values.  (Measured at 12 to 24 items.)
-constexpr int items_per_thread(int key_bytes, int value_bytes) {
-  if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS8 : ILGPU_HIP_SORT_ITEMS;
-  if (value_bytes == 16) return 8;
-  const int registers = (key_bytes == 8 ? 2 : 1) + (value_bytes == 8 ? 2 : 1);
-  return registers == 2 ? 20 : registers == 3 ? ILGPU_HIP_SORT_PAIR_ITEMS3 : 14;
-}
-constexpr int tile_keys(int key_bytes, int value_bytes, int block) {
-  return block * items_per_thread(key_bytes, value_bytes);
-}
-
-// How raw key bits map to unsigned bits that sort in the requested order.
-// ordered(k) = k ^ xor_mask ^ (lsr(~k, bits-1) & reference_term) ^ (asr(k, bits-1) & total_term):
-// branch-free for every mode.  reference_term is 1 for the float order of the
-// reference (RadixSortOperations.tt:81-89 as written: the complement mask is a
-// LOGICAL shift of ~bits, i.e. 1 for non-negative values and 0 otherwise);
-// total_term is all bits below the sign for IEEE totalOrder (negative values
-// have them flipped); both are 0 for integer keys.
-struct KeyXform {
-  uint64_t xor_mask;
-  uint64_t reference_term;
-  uint64_t total_term;
-};
-
-template <typename K>
-__device__ __forceinline__ K key_term(K k, const KeyXform& xf) {
-  constexpr int kBits = sizeof(K) * 8;
-  using S = typename std::make_signed<K>::type;
-  return (K)(((K)((K)(~k) >> (kBits - 1)) & (K)xf.reference_term) ^
-             ((K)((S)k >> (kBits - 1)) & (K)xf.total_term));
-}
-
-template <typename K>
-__device__ __forceinline__ K ordered_bits(K k, const KeyXform& xf) {
-  return (K)(k ^ (K)xf.xor_mask ^ key_term(k, xf));
-}
-
-template <typename K>
-__device__ __forceinline__ uint32_t digit_of(K k, const KeyXform& xf, int shift) {
-  return (uint32_t)(ordered_bits(k, xf) >> shift) & (kRadix - 1);
-}
-
-// Inverse of ordered_bits.  The per-key term depends on the key's sign bit
-// only and never changes it, so u = o ^ xor_mask has the sign bit of the key
-// and the same term taken from u gives the key back.
-template <typename K>
-__device__ __forceinline__ K raw_bits(K o, const KeyXform& xf) {
-  const K u = (K)(o ^ (K)xf.xor_mask);
-  return (K)(u ^ key_term(u, xf));
-}
-
-constexpr uint32_t kNoHotDigit = 0xFFFFFFFFu;
-constexpr int kMaxHot = 4;
-// Device-resident description of the passes, written by plan_kernel.
-struct SortPlan {
-  uint32_t skip[kMaxPasses];        // digit identical for all keys
-  uint32_t src_is_alt[kMaxPasses];  // pass reads the alternate buffer
-  // Up to kMaxHot digits that each hold an eighth of the keys or more, most
-  // frequent first; unused entries are kNoHotDigit.
-  uint32_t hot[kMaxPasses][kMaxHot];
-  uint32_t first_executed;          // index of the first pass that runs
-  uint32_t last_executed;           // index of the last pass that runs
-  uint32_t executed;                // number of passes that run
-  uint32_t final_in_alt;            // result sits in the alternate buffer
-};
-
-// ---- histogram of all digit positions ------------------------------------
-template <typename K>
-__global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
-    const K* __restrict__ keys, int64_t n, KeyXform xf, int passes,
-    int replica_shift, uint32_t* __restrict__ global_hist) {
-  using V = typename Vec16<K>::type;
-  constexpr int VN = Vec16<K>::N;
-  extern __shared__ uint32_t s_hist[];  // [passes][256][replicas]
-  const int words = (passes * kRadix) << replica_shift;
-  for (int i = threadIdx.x; i < words; i += kHistBlock) s_hist[i] = 0u;
-  __syncthreads();
-
-  const uint32_t replica = threadIdx.x & ((1u << replica_shift) - 1u);
-  const bool has_term = (xf.reference_term | xf.total_term) != 0;  // float keys
-  auto count = [&](K k) {
-    K o = (K)(k ^ (K)xf.xor_mask);
-    if (has_term) o ^= key_term(k, xf);
-#pragma unroll
-    for (int p = 0; p < (int)sizeof(K); ++p) {
-      const uint32_t d = (uint32_t)(o >> (8 * p)) & (kRadix - 1);
-      atomicAdd(&s_hist[((p * kRadix + d) << replica_shift) + replica], 1u);
-    }
-  };
-
-  const uintptr_t addr = reinterpret_cast<uintptr_t>(keys);
-  int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(K));
-  if (head > n) head = n;
-  const V* body = reinterpret_cast<const V*>(keys + head);
-  const int64_t nvec = (n - head) / VN;
-  const int64_t tail_start = head + nvec * VN;
-  const int64_t stride = (int64_t)gridDim.x * kHistBlock;
-  int64_t i = (int64_t)blockIdx.x * kHistBlock + threadIdx.x;
-  for (; i + stride < nvec; i += 2 * stride) {
-    V a = body[i];
-    V b = body[i + stride];
-#pragma unroll
-    for (int k = 0; k < VN; ++k) count(a[k]);
-#pragma unroll
-    for (int k = 0; k < VN; ++k) count(b[k]);
-  }
-  for (; i < nvec; i += stride) {
-    V a = body[i];
-#pragma unroll
-    for (int k = 0; k < VN; ++k) count(a[k]);
-  }
-  if (blockIdx.x == 0) {
-    const int64_t extra = head + (n - tail_start);
-    if ((int64_t)threadIdx.x < extra) {
-      const int64_t idx = (int64_t)threadIdx.x < head
-                              ? (int64_t)threadIdx.x
-                              : tail_start + ((int64_t)threadIdx.x - head);
-      count(keys[idx]);
-    }
-  }
-  __syncthreads();
-
-  const int replicas = 1 << replica_shift;
-  for (int b = threadIdx.x; b < passes * kRadix; b += kHistBlock) {
-    uint32_t c = 0;
-    for (int r = 0; r < replicas; ++r)
-      c += s_hist[(b << replica_shift) + ((r + b) & (replicas - 1))];
-    if (c != 0) atomicAdd(&global_hist[b], c);
-  }
-}
-
-// ---- plan: exclusive digit offsets, skipped passes, buffer parity ---------
-__global__ __launch_bounds__(kRadix) void plan_kernel(
-    const uint32_t* __restrict__ global_hist, uint32_t* __restrict__ excl,
-    SortPlan* __restrict__ plan, int passes, uint32_t n) {
-  __shared__ uint32_t s_wave[kRadix / kWaveSize];
-  __shared__ int s_trivial;
-  __shared__ unsigned long long s_hot[kMaxHot];  // count << 8 | digit, most frequent first
-  const int d = threadIdx.x;
-  const int lane = d & (kWaveSize - 1);
-  const int wave = d / kWaveSize;
-  uint32_t parity = 0, executed = 0, first = passes, last = passes;
-  for (int p = 0; p < passes; ++p) {
-    if (d < kMaxHot) s_hot[d] = 0ull;
-    if (d == 0) s_trivial = 0;
-    __syncthreads();
-    const uint32_t c = global_hist[p * kRadix + d];
-    if (c == n) s_trivial = 1;
-    // A digit qualifies with an eighth of the keys (two lanes of a
-    // sub-tile row on average); kMaxHot rounds of "largest below the previous
-    // one" order the most frequent ones.
-    const unsigned long long mine = ((unsigned long long)c << 8) | (unsigned long long)d;
-    const bool frequent = (uint64_t)c * 8 >= (uint64_t)n;
-    for (int h = 0; h < kMaxHot; ++h) {
-      if (frequent && (h == 0 || mine < s_hot[h - 1])) atomicMax(&s_hot[h], mine);
-      __syncthreads();
-    }
-    uint32_t inc = c;
-#pragma unroll
-    for (int s = 1; s < kWaveSize; s <<= 1) {
-      const uint32_t o = shfl_up(inc, s);
-      if (lane >= s) inc += o;
-    }
-    if (lane == kWaveSize - 1) s_wave[wave] = inc;
-    __syncthreads();
-    uint32_t off = 0;
-    for (int w = 0; w < wave; ++w) off += s_wave[w];
-    excl[p * kRadix + d] = off + inc - c;
-    const bool trivial = s_trivial != 0;
-    if (d == 0) {
-      plan->skip[p] = trivial ? 1u : 0u;
-      plan->src_is_alt[p] = parity;
-      for (int h = 0; h < kMaxHot; ++h)
-        plan->hot[p][h] = s_hot[h] != 0ull ? (uint32_t)(s_hot[h] & 0xFFull) : kNoHotDigit;
-    }
-    if (!trivial) {
-      if (executed == 0) first = p;
-      last = p;
-      parity ^= 1u;
-      ++executed;
-    }
-    __syncthreads();
-  }
-  if (d == 0) {
-    plan->first_executed = first;
-    plan->last_executed = last;
-    plan->executed = executed;
-    plan->final_in_alt = parity;
-  }
-}
-
-// ---- onesweep pass ---------------------------------------------------------
-// Ranking.  A block's tile is cut into sub-tiles, one per wave; lane l of wave
-// w holds items w*64*kItems + j*64 + l, j = 0 .. kItems-1, so memory order
-// inside a sub-tile is (row j, lane) and a row is one 256-byte load.  Every
-// (wave, digit) pair owns one 32-bit LDS counter.  For row j every lane adds
-// one to the counter of its digit with a returning LDS atomic; the value that
-// comes back is the key's rank among the keys of that digit in the sub-tile.
-//
-// That the rank follows memory order rests on two properties of the LDS:
-// instructions of one wave execute in issue order (rows chain through the
-// counters without barriers), and the lanes of ONE atomic instruction that
-// meet in one address are served in ascending lane order.  The second is a
-// property of this hardware (gfx950), not of the programming model; it is
-// checked on the device by ilgpu_hip_selftest_lds_atomic_order and, end to
-// end, by every stability test of the pair sorts.  With it the pass is stable
-// at one LDS operation per key and no cross-lane arithmetic.
-template <int KEY_BYTES, int VALUE_BYTES, int BLOCK> struct SortTile {
-  static constexpr int kSubTiles = BLOCK / kSubLanes;
-  static constexpr int kCounterWords = kSubTiles * kRadix;
-  static constexpr int kCounterBytes = kCounterWords * 4;
-  static constexpr int kItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
-  static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES, BLOCK);
-  static constexpr int kSubTileKeys = kSubLanes * kItems;
-  static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
-  static constexpr int kStageBytes =
-      kCounterBytes > kKeyStageBytes ? kCounterBytes : kKeyStageBytes;
-};
-
-template <int KEY_BYTES, int ITEMS, bool FULL>
-__device__ __forceinline__ void load_tile_keys(
-    const typename KeyOf<KEY_BYTES>::type* __restrict__ src, int64_t tile_base,
-    int valid, int first_local,
-    typename KeyOf<KEY_BYTES>::type (&key)[ITEMS]) {
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    const int local = first_local + j * kSubLanes;
-    if (FULL || local < valid) key[j] = src[tile_base + local];
-    else key[j] = 0;
-  }
-}
-
-// Waves per SIMD the pass kernel is compiled for: sixteen waves per CU, as two
-// 512-thread blocks or one 1024-thread block.  That bounds a thread at 128
-// registers (36 keys and 18 registers of packed ranks in a keys-only sort;
-// fewer items when values ride along) and the blocks of a CU at 160 KiB of
-// LDS together (a 36-key tile stages 72 KiB per 512 threads).
-#ifndef ILGPU_HIP_SORT_WAVES_PER_EU
-#define ILGPU_HIP_SORT_WAVES_PER_EU 4
-#endif
-
-// Tile of a group's k-th draw: its chunks are g, g + 8, g + 16, ... of
-// 2^chunk_shift consecutive tiles.
-__device__ __forceinline__ int ticket_tile(uint32_t k, uint32_t g, int chunk_shift) {
-  const uint32_t chunk = (k >> chunk_shift) * kTicketGroups + g;
-  return (int)((chunk << chunk_shift) + (k & ((1u << chunk_shift) - 1u)));
-}
-
-// Sorts one tile by the digit of `pass` and scatters it.
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT, int BLOCK>
-__device__ __forceinline__ void sort_tile(
-    typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
-    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys,
-    typename KeyOf<KEY_BYTES>::type* __restrict__ dst_keys,
-    const typename ValueOf<VALUE_BYTES>::type* __restrict__ src_vals,
-    typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
-    int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
-    const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
-    unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan,
-    const uint32_t (&hot)[kMaxHot], uint32_t spin_limit, bool in_raw, bool out_raw) {
-  using K = typename KeyOf<KEY_BYTES>::type;
-  using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
-  constexpr int kItems = TileCfg::kItems;
-  constexpr int kSubTiles = TileCfg::kSubTiles;
-  constexpr bool kPairs = VALUE_BYTES > 0;
-  constexpr int kValuesPerRound =
-      kPairs ? TileCfg::kStageBytes / (VALUE_BYTES > 0 ? VALUE_BYTES : 1) : 1;
-  constexpr int kRounds =
-      kPairs ? (TileCfg::kTile + kValuesPerRound - 1) / kValuesPerRound : 0;
-  static_assert(kItems % 2 == 0 && TileCfg::kTile <= 65536,
-                "ranks and tile positions are packed two to a register");
-  static_assert(kItems * kSubLanes < 65536, "a sub-tile's digit count fits 16 bits");
-
-  // Counter of (sub-tile, digit): keys of that digit in the rows ranked so far.
-  uint32_t* s_counter = reinterpret_cast<uint32_t*>(s_stage);
-  K* s_keys = reinterpret_cast<K*>(s_stage);
-  Val* s_vals = reinterpret_cast<Val*>(s_stage);
-
-  // The thread index is made opaque per tile (and again for the write-out):
-  // otherwise every per-item index derived from it is hoisted out of the
-  // tile loop and held in a register of its own, dozens of them.
-  int tid = threadIdx.x;
-  asm volatile("" : "+v"(tid));
-  const int lane = tid & (kWaveSize - 1);
-  const int wave = tid / kWaveSize;
-  const int sub = wave;                     // sub-tile index in the block
-  const int first_local = sub * TileCfg::kSubTileKeys + lane;
-  const int shift = pass * 8;
-
-
-  // Float keys travel between the passes in their ordered form: the first
-  // pass that runs converts them as it ranks them (in_raw), the last one
-  // converts them back as it writes them (out_raw), and in between a digit is
-  // a shift and a mask.  Other keys keep their bits; their order is one xor.
-  // (A pass that finds them converted applies the identity: no mask, no term.)
-  KeyXform xf_in = xf;
-  if (!in_raw) xf_in = KeyXform{0, 0, 0};
-  auto digit = [&](K k) -> uint32_t {
-    if constexpr (FLOAT_KEYS) return (uint32_t)(k >> shift) & (kRadix - 1);
-    else return (uint32_t)((K)(k ^ (K)xf.xor_mask) >> shift) & (kRadix - 1);
-  };
-  // Keys past the end of the input take digit 255; they come last in memory
-  // order, so they rank behind every real key and are dropped on write-out.
-  auto item_digit = [&](int j) -> uint32_t {
-    return (FULL || first_local + j * kSubLanes < valid) ? digit(key[j])
-                                                          : (uint32_t)(kRadix - 1);
-  };
-
-  Val val[kPairs ? kItems : 1];
-  if constexpr (kPairs) {
-#pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-      const int local = first_local + j * kSubLanes;
-      if (FULL || local < valid) {
-        if (make_index) {
-          if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)(tile_base + local);
-          else if constexpr (VALUE_BYTES == 8) val[j] = (Val)(uint64_t)(tile_base + local);
-        } else {
-          val[j] = src_vals[tile_base + local];
-        }
-      }
-    }
-  }
-
-  // Rank inside the sub-tile, later position inside the tile: 16 bits each.
-  uint32_t* my_counters = s_counter + sub * kRadix;
-  uint32_t packed[kItems / 2];
-  // HOT: some digits hold a large share of the keys each (known from the
-  // global histogram).  Their keys would all meet in one counter, and LDS
-  // serialises the atomics of a wave to one address; they are ranked by one
-  // ballot per such digit instead and only the other keys go through the
-  // counters.
-  uint32_t hot_count[kMaxHot] = {};  // keys of each hot digit in this sub-tile so far
-  // Rows are ranked in groups: the LDS operations of a group are issued back
-  // to back and their results consumed together, so a wave waits for one LDS
-  // round trip per group, not per row.
-  // (Pairs hold their values in registers too and take smaller groups.)
-  constexpr int kGroup = kPairs ? ILGPU_HIP_SORT_PAIR_RANK_GROUP : ILGPU_HIP_SORT_RANK_GROUP;
-  static_assert(kGroup % 2 == 0, "ranks are packed in pairs");
-#pragma unroll
-  for (int j0 = 0; j0 < kItems; j0 += kGroup) {
-    uint32_t fetched[kGroup];   // what the LDS returned for the row
-    uint32_t offset[kGroup];    // added to it: lane index of a one-digit row
-    bool broadcast[kGroup];     // wave-uniform: take lane 0's result
-#pragma unroll
-    for (int g = 0; g < kGroup; ++g) {
-      const int j = j0 + g;
-      if (j >= kItems) break;
-      const uint32_t d = item_digit(j);
-      fetched[g] = 0;
-      offset[g] = 0;
-      broadcast[g] = false;
-      bool through_counter = true;
-      if constexpr (HOT) {
-#pragma unroll
-        for (int h = 0; h < kMaxHot; ++h) {
-          if (hot[h] == kNoHotDigit) continue;  // wave-uniform
-          const bool is_hot = d == hot[h];
-          const uint64_t hot_lanes = __ballot(is_hot);
-          if (is_hot) {
-            offset[g] = hot_count[h] + (uint32_t)mbcnt(hot_lanes);
-            through_counter = false;
-          }
-          hot_count[h] += (uint32_t)__popcll(hot_lanes);
-        }
-      } else {
-        // Keys that arrive in runs put one digit into whole rows of a
-        // sub-tile; the 64 atomics of such a row would meet in one word and
-        // serialise.  In a row that is all one digit only lane 0 adds (the
-        // whole row at once) and the others take its result plus their lane
-        // index.  Passes with dominant digits leave the check out: the
-        // ballots above already took their frequent digits.
-        const uint32_t row_digit = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
-        broadcast[g] = __ballot(d == row_digit) == ~0ull;
-        if (broadcast[g]) {
-          offset[g] = (uint32_t)lane;
-          through_counter = lane == 0;
-        }
-      }
-      if (through_counter)
-        fetched[g] = __hip_atomic_fetch_add(my_counters + d,
-                                            broadcast[g] ? (uint32_t)kSubLanes : 1u,
-                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-#pragma unroll
-    for (int g = 0; g < kGroup; ++g) {
-      const int j = j0 + g;
-      if (j >= kItems) break;
-      uint32_t rank = fetched[g];
-      if constexpr (!HOT) {
-        if (broadcast[g]) rank = (uint32_t)__builtin_amdgcn_readfirstlane((int)rank);
-      }
-      rank += offset[g];
-      if (j % 2 == 0) packed[j / 2] = rank;
-      else packed[j / 2] |= rank << 16;
-    }
-    // Pin the packed ranks here: left alone, the compiler sinks the rank
-    // arithmetic of all rows to where the ranks are used and keeps two live
-    // registers per key until then.
-#pragma unroll
-    for (int g = 0; g < kGroup; g += 2)
-      if (j0 + g < kItems) asm volatile("" : "+v"(packed[(j0 + g) / 2]));
-  }
-  if constexpr (HOT) {
-#pragma unroll
-    for (int h = 0; h < kMaxHot; ++h)  // these counters are untouched so far: still zero
-      if (hot[h] != kNoHotDigit && lane == 0) my_counters[hot[h]] = hot_count[h];
-  }
-  __syncthreads();
-
-  // One thread per digit: totals over the sub-tiles, look-back over the tiles.
-  uint32_t count = 0, inc = 0;
-  uint32_t* tile_status = status + (int64_t)tile * kRadix;
-  if (tid < kRadix) {
-#pragma unroll
-    for (int s = 0; s < kSubTiles; ++s) count += s_counter[s * kRadix + tid];
-    __hip_atomic_store(&tile_status[tid],
-                       tile == 0 ? status_prefix(count) : status_aggregate(count),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    inc = count;
-#pragma unroll
-    for (int s = 1; s < kWaveSize; s <<= 1) {
-      const uint32_t o = shfl_up(inc, s);
-      if (lane >= s) inc += o;
-    }
-    if (lane == kWaveSize - 1) s_scan[wave] = inc;
-  }
-  __syncthreads();
-  // Digit threads: run starts, and the first step of the look-back is put in
-  // flight; it is consumed after the keys are staged, so its round trip
-  // overlaps the position and staging work of the whole block.
-  uint32_t digit_start = 0;
-  uint32_t first_step[kLookback];
-  if (tid < kRadix) {
-    digit_start = inc - count;
-    for (int w = 0; w < wave; ++w) digit_start += s_scan[w];
-    // Tile-local position of the first key of every (sub-tile, digit) run.
-    {
-      uint32_t run = digit_start;
-#pragma unroll
-      for (int s = 0; s < kSubTiles; ++s) {
-        const uint32_t t = s_counter[s * kRadix + tid];
-        s_counter[s * kRadix + tid] = run;
-        run += t;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < kLookback; ++u) {
-      const int idx = tile - 1 - u < 0 ? 0 : tile - 1 - u;
-      first_step[u] = __hip_atomic_load(&status[(int64_t)idx * kRadix + tid],
-                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  __syncthreads();
-
-  // Tile-local position of every key; afterwards the counters are dead and
-  // the same LDS bytes stage the keys in digit order.
-#pragma unroll
-  for (int j = 0; j < kItems; j += 2) {
-    const uint32_t p0 = my_counters[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
-    const uint32_t p1 = my_counters[item_digit(j + 1)] + (packed[j / 2] >> 16);
-    packed[j / 2] = p0 | (p1 << 16);
-    if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
-  }
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < kItems; ++j)
-    s_keys[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = key[j];
-
-  if (tid < kRadix) {
-    // Keys with this digit in earlier tiles: walk back over the status words,
-    // kLookback tiles per step.  The loads of a step are unconditional (index
-    // clamped) so that they are in flight together; positions in front of
-    // tile 0 read as an empty inclusive prefix.
-    uint32_t before = 0;
-    bool done = tile == 0;
-    bool preloaded = true;
-    for (int t = tile - 1; !done; t -= kLookback) {
-      uint32_t s[kLookback];
-#pragma unroll
-      for (int u = 0; u < kLookback; ++u) {
-        if (preloaded) {
-          s[u] = first_step[u];
-        } else {
-          const int idx = t - u < 0 ? 0 : t - u;
-          s[u] = __hip_atomic_load(&status[(int64_t)idx * kRadix + tid],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-      }
-      preloaded = false;
-#pragma unroll
-      for (int u = 0; u < kLookback; ++u)
-        if (t - u < 0) s[u] = status_prefix(0u);
-#pragma unroll
-      for (int u = 0; u < kLookback; ++u) {
-        if (done) continue;
-        uint32_t polls = 0;
-        while (s[u] == 0u) {
-          if (polls++ >= spin_limit) {
-            // Nobody has published tile t - u: its owner may not be running.
-            // Count this thread's digit in that tile from the source keys (a
-            // full tile: it precedes this one) and go on as if the tile had
-            // published its own count.  Slow, and never needed while every
-            // group of blocks is resident.
-            const K* other = src_keys + (int64_t)(t - u) * TileCfg::kTile;
-            uint32_t c = 0;
-#pragma unroll 4
-            for (int i = 0; i < TileCfg::kTile; ++i) {
-              K k = other[i];
-              if constexpr (FLOAT_KEYS) k = ordered_bits(k, xf_in);
-              c += digit(k) == (uint32_t)tid;
-            }
-            s[u] = status_aggregate(c);
-            break;
-          }
-          __builtin_amdgcn_s_sleep(1);
-          s[u] = __hip_atomic_load(&status[(int64_t)(t - u) * kRadix + tid],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        before += status_value(s[u]);
-        done = !status_is_aggregate(s[u]);
-      }
-    }
-    if (tile > 0)
-      __hip_atomic_store(&tile_status[tid], status_prefix(before + count),
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_global_off[tid] = excl[pass * kRadix + tid] + before - digit_start;
-  }
-  __syncthreads();
-
-  uint32_t gpos[kPairs ? kItems : 1];
-  asm volatile("" : "+v"(tid));
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    const int i = j * BLOCK + tid;
-    if (FULL || i < valid) {
-      const K k = s_keys[i];
-      const uint32_t g = s_global_off[digit(k)] + (uint32_t)i;
-      if constexpr (FLOAT_KEYS) dst_keys[g] = out_raw ? raw_bits(k, xf) : k;
-      else dst_keys[g] = k;
-      if constexpr (kPairs) gpos[j] = g;
-    }
-    constexpr int kWriteGroup = kPairs ? ILGPU_HIP_SORT_PAIR_WRITE_GROUP : ILGPU_HIP_SORT_WRITE_GROUP;
-    if (j % kWriteGroup == kWriteGroup - 1) __builtin_amdgcn_sched_barrier(0);
-  }
-
-  if constexpr (kPairs) {
-#pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-      const uint32_t lo = (uint32_t)r * kValuesPerRound;
-      __syncthreads();  // the stage buffer is free again
-#pragma unroll
-      for (int j = 0; j < kItems; ++j) {
-        const uint32_t pos = j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16;
-        if (pos - lo < (uint32_t)kValuesPerRound) s_vals[pos - lo] = val[j];
-      }
-      __syncthreads();
-#pragma unroll
-      for (int j = 0; j < kItems; ++j) {
-        const uint32_t i = (uint32_t)(j * BLOCK + tid);
-        if ((FULL || i < (uint32_t)valid) && i - lo < (uint32_t)kValuesPerRound)
-          dst_vals[gpos[j]] = s_vals[i - lo];
-      }
-    }
-  }
-}
-
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, int BLOCK>
-__global__ __launch_bounds__(BLOCK, ILGPU_HIP_SORT_WAVES_PER_EU)
-void onesweep_kernel(
-    typename KeyOf<KEY_BYTES>::type* keys_a,
-    typename KeyOf<KEY_BYTES>::type* keys_b,
-    typename ValueOf<VALUE_BYTES>::type* vals_a,
-    typename ValueOf<VALUE_BYTES>::type* vals_b, int64_t n, int pass,
-    KeyXform xf, const uint32_t* __restrict__ excl, uint32_t* status,
-    uint32_t* ticket, const SortPlan* __restrict__ plan, int num_tiles,
-    int values_from_index, int chunk_shift, uint32_t spin_limit) {
-  using K = typename KeyOf<KEY_BYTES>::type;
-  using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
-  constexpr int kTile = TileCfg::kTile;
-  constexpr int kItems = TileCfg::kItems;
-
-  __shared__ __attribute__((aligned(16))) unsigned char s_stage[TileCfg::kStageBytes];
-  __shared__ uint32_t s_global_off[kRadix];
-  __shared__ uint32_t s_scan[kRadix / kWaveSize];
-  __shared__ int s_tile;
-
-  if (plan->skip[pass]) return;
-  const bool src_alt = plan->src_is_alt[pass] != 0;
-  uint32_t hot[kMaxHot];
-#pragma unroll
-  for (int h = 0; h < kMaxHot; ++h) hot[h] = plan->hot[pass][h];
-  const K* src_keys = src_alt ? keys_b : keys_a;
-  K* dst_keys = src_alt ? keys_a : keys_b;
-  const Val* src_vals = src_alt ? vals_b : vals_a;
-  Val* dst_vals = src_alt ? vals_a : vals_b;
-  const bool make_index = VALUE_BYTES > 0 && values_from_index &&
-                          plan->first_executed == (uint32_t)pass;
-  const bool in_raw = plan->first_executed == (uint32_t)pass;
-  const bool out_raw = plan->last_executed == (uint32_t)pass;
-  const int tid = threadIdx.x;
-  const int first_local = (tid / kSubLanes) * TileCfg::kSubTileKeys + tid % kSubLanes;
-
-  auto valid_keys = [&](int t) -> int {
-    const int64_t remaining = n - (int64_t)t * kTile;
-    return remaining >= kTile ? kTile : (remaining > 0 ? (int)remaining : 0);
-  };
-
-  // Tickets: group g (= blockIdx % 8) owns the chunks g, g + 8, g + 16, ... of
-  // 2^chunk_shift consecutive tiles and draws their tiles in order from its
-  // own counter.  Unlike a single counter this does not start tiles in index
-  // order across groups: a tile can find that a predecessor owned by another
-  // group has not been started, and if that group had no resident block it
-  // would wait for ever.  The look-back therefore never waits without bound:
-  // after spin_limit polls of an empty word it counts the tile's digit itself
-  // (sort_tile), so every block finishes whatever the other blocks do.
-  // A block draws its next tile only when it is about to start it: the time
-  // between a tile's ticket and the publication of its digit counts is what
-  // every later tile's look-back waits for.  (Drawing it earlier, to load the
-  // next keys during the look-back and the write-out, measured 3 to 12 % slower,
-  // with the global ticket and again with the per-group ones.)  The key loads
-  // fly while the ranking counters are cleared.
-  while (true) {
-    if (tid == 0) {
-      const uint32_t g = blockIdx.x % (uint32_t)kTicketGroups;
-      s_tile = ticket_tile(atomicAdd(ticket + g * kTicketStride, 1u), g, chunk_shift);
-    }
-    __syncthreads();  // also: the previous tile's staged keys have been read
-    const int tile = s_tile;
-    if (tile >= num_tiles) break;
-    const int64_t tile_base = (int64_t)tile * kTile;
-    const int valid = valid_keys(tile);
-    // Three instantiations of the tile code: full tiles with and without
-    // dominant digits, and the tail tile (bounds-checked; the dominant-digit
-    // form serves it either way: without such digits every key goes through
-    // the counters).  Each loads its keys itself, so that the loads, the
-    // clearing of the counters and the ranking are one straight line and the
-    // rows are ranked as their keys arrive.
-    auto run = [&](auto full, auto with_hot) {
-      constexpr bool kFull = decltype(full)::value;
-      constexpr bool kHot = decltype(with_hot)::value;
-      K key[kItems];
-      load_tile_keys<KEY_BYTES, kItems, kFull>(src_keys, tile_base, valid, first_local, key);
-      if constexpr (FLOAT_KEYS) {
-        if (in_raw) {
-#pragma unroll
-          for (int j = 0; j < kItems; ++j) key[j] = ordered_bits(key[j], xf);
-        }
-      }
-      {  // clear the ranking counters
-        uint4* z = reinterpret_cast<uint4*>(s_stage);
-        for (int i = tid; i < TileCfg::kCounterBytes / 16; i += BLOCK)
-          z[i] = make_uint4(0u, 0u, 0u, 0u);
-      }
-      __syncthreads();
-      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot, BLOCK>(
-          key, src_keys, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl,
-          status, make_index, s_stage, s_global_off, s_scan, hot, spin_limit, in_raw, out_raw);
-    };
-    if (valid != kTile) run(std::false_type{}, std::true_type{});
-    else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
-    else run(std::true_type{}, std::true_type{});
-  }
-}
 
 // ---- device check of the LDS property the ranking rests on -------------------
 // Every wave keeps 256 counters and plays `rows` ranking rows on pseudo-random
@@ -853,227 +54,6 @@ __global__ __launch_bounds__(kSortBlock) void lds_atomic_order_kernel(
   if (wrong != 0) atomicAdd(mismatches, wrong);
 }
 
-// ---- finish ----------------------------------------------------------------
-template <int KEY_BYTES, int VALUE_BYTES>
-__global__ __launch_bounds__(256) void finish_kernel(
-    typename KeyOf<KEY_BYTES>::type* keys_a,
-    const typename KeyOf<KEY_BYTES>::type* keys_b,
-    typename ValueOf<VALUE_BYTES>::type* vals_a,
-    const typename ValueOf<VALUE_BYTES>::type* vals_b, int64_t n,
-    const SortPlan* __restrict__ plan, int values_from_index) {
-  using Val = typename ValueOf<VALUE_BYTES>::type;
-  const bool copy_back = plan->final_in_alt != 0;
-  const bool fill_index =
-      VALUE_BYTES > 0 && values_from_index && plan->executed == 0;
-  if (!copy_back && !fill_index) return;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += stride) {
-    if (copy_back) {
-      keys_a[i] = keys_b[i];
-      if constexpr (VALUE_BYTES > 0) vals_a[i] = vals_b[i];
-    } else {
-      if constexpr (VALUE_BYTES == 4) vals_a[i] = (Val)(uint32_t)i;
-      else if constexpr (VALUE_BYTES == 8) vals_a[i] = (Val)(uint64_t)i;
-    }
-  }
-}
-
-// ---- host side -------------------------------------------------------------
-std::atomic<uint32_t> g_spin_limit{kDefaultSpinLimit};
-std::atomic<int32_t> g_large_min_tiles_per_cu{-1};  // negative: the defaults above
-
-struct TempLayout {
-  int64_t alt_keys, alt_vals, excl, plan, zero_begin, hist, tickets, status,
-      status_stride, total;
-  int64_t tiles;
-};
-
-// Layout for tiles of `block` threads.  Temp views are sized for the small
-// block (more tiles, more status words); the large block's layout fits inside.
-TempLayout make_layout(int64_t n, int key_bytes, int value_bytes, int block = kSortBlock) {
-  TempLayout L;
-  const int64_t tile = tile_keys(key_bytes, value_bytes, block);
-  L.tiles = div_up(n, tile);
-  int64_t off = 0;
-  L.alt_keys = off; off += align_up(n * key_bytes, 256);
-  L.alt_vals = off; off += align_up(n * value_bytes, 256);
-  L.excl = off; off += kMaxPasses * kRadix * 4;
-  L.plan = off; off += 256;
-  L.zero_begin = off;
-  L.hist = off; off += kMaxPasses * kRadix * 4;
-  L.tickets = off; off += kMaxPasses * kTicketGroups * kTicketStride * 4;
-  L.status = off;
-  L.status_stride = L.tiles * kRadix * 4;
-  off += L.status_stride * key_bytes;  // one status array per pass
-  L.total = off;
-  return L;
-}
-
-KeyXform make_xform(int32_t key_type, int32_t flags) {
-  const int bits = elem_size(key_type) * 8;
-  const uint64_t all = bits == 64 ? ~0ull : ((1ull << bits) - 1ull);
-  const uint64_t sign = 1ull << (bits - 1);
-  KeyXform xf{0, 0, 0};
-  switch (key_type) {
-    case ILGPU_HIP_I8: case ILGPU_HIP_I16: case ILGPU_HIP_I32: case ILGPU_HIP_I64:
-      xf.xor_mask = sign;
-      break;
-    case ILGPU_HIP_F16: case ILGPU_HIP_F32: case ILGPU_HIP_F64:
-      if (flags & ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER) {
-        xf.xor_mask = sign;
-        xf.total_term = sign - 1ull;
-      } else {
-        // Half: (uint)~bits >> 15 keeps the sign-extended upper ones, so bits
-        // 1..15 are always flipped (RadixSortOperations.tt:77-80).
-        xf.xor_mask = key_type == ILGPU_HIP_F16 ? 0xFFFEull : sign;
-        xf.reference_term = 1ull;
-      }
-      break;
-    default:
-      break;
-  }
-  if (flags & ILGPU_HIP_SORT_DESCENDING) xf.xor_mask ^= all;
-  return xf;
-}
-
-// The passes of one sort with tiles of BLOCK threads.
-template <int KEY_BYTES, int VALUE_BYTES, int BLOCK>
-int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L, char* base,
-                      const KeyXform& xf, int cus) {
-  using K = typename KeyOf<KEY_BYTES>::type;
-  using Val = typename ValueOf<VALUE_BYTES>::type;
-  K* keys_a = static_cast<K*>(a.keys);
-  K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
-  Val* vals_a = static_cast<Val*>(a.values);
-  Val* vals_b = reinterpret_cast<Val*>(base + L.alt_vals);
-  uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
-  SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
-  uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
-  const int passes = KEY_BYTES;
-  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
-  const bool float_keys = (xf.reference_term | xf.total_term) != 0;
-  auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false, BLOCK>;
-  if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
-    if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true, BLOCK>;
-  }
-  // Resident blocks per CU of this instantiation: asked once per device and
-  // kernel (the query costs microseconds, which small sorts would feel).
-  static std::atomic<int> cached_per_cu[kMaxCachedDevices][2];  // per instantiation
-  const int device = current_device();
-  std::atomic<int>* cached =
-      device >= 0 && device < kMaxCachedDevices ? &cached_per_cu[device][float_keys ? 1 : 0]
-                                                : nullptr;
-  int per_cu = cached ? cached->load(std::memory_order_relaxed) : 0;
-  if (per_cu == 0) {
-    ILGPU_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
-        &per_cu, pass_kernel, BLOCK, 0));
-    if (per_cu < 1) per_cu = 1;
-    if (cached) cached->store(per_cu, std::memory_order_relaxed);
-  }
-  int64_t grid = (int64_t)cus * per_cu;
-  if (grid > L.tiles) grid = L.tiles;
-  // Chunks as long as leave every block of the grid a tile of its own in the
-  // first round (short inputs: single tiles, handed out round-robin).
-  int chunk_shift = 0;
-  while (chunk_shift < kMaxChunkShift && (grid << (chunk_shift + 1)) <= L.tiles) ++chunk_shift;
-  const uint32_t spin_limit = g_spin_limit.load(std::memory_order_relaxed);
-  for (int p = 0; p < passes; ++p) {
-    uint32_t* status =
-        reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
-    {
-      ProfileScope scope(stream, "sort_onesweep");
-      hipLaunchKernelGGL(pass_kernel,
-                         dim3((unsigned)grid), dim3(BLOCK), 0, stream,
-                         keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
-                         status, tickets + p * kTicketGroups * kTicketStride, plan, (int)L.tiles,
-                         from_index, chunk_shift, spin_limit);
-    }
-    ILGPU_HIP_CHECK(hipGetLastError());
-  }
-  return ILGPU_HIP_SUCCESS;
-}
-
-template <int KEY_BYTES, int VALUE_BYTES>
-int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
-  using K = typename KeyOf<KEY_BYTES>::type;
-  using Val = typename ValueOf<VALUE_BYTES>::type;
-  const int cus = device_cu_count();
-  int64_t min_tiles_per_cu = g_large_min_tiles_per_cu.load(std::memory_order_relaxed);
-  if (min_tiles_per_cu < 0)
-    min_tiles_per_cu = VALUE_BYTES > 0 ? kLargeMinTilesPerCuPairs : kLargeMinTilesPerCuKeys;
-  const bool use_large =
-      div_up(a.n, (int64_t)tile_keys(KEY_BYTES, VALUE_BYTES, kSortBlockLarge)) >=
-      min_tiles_per_cu * cus;
-  const TempLayout L =
-      make_layout(a.n, KEY_BYTES, VALUE_BYTES, use_large ? kSortBlockLarge : kSortBlock);
-  char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)a.temp, 256));
-  K* keys_a = static_cast<K*>(a.keys);
-  K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
-  Val* vals_a = static_cast<Val*>(a.values);
-  Val* vals_b = reinterpret_cast<Val*>(base + L.alt_vals);
-  uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
-  SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
-  uint32_t* hist = reinterpret_cast<uint32_t*>(base + L.hist);
-  const KeyXform xf = make_xform(a.key_type, a.flags);
-  const int passes = KEY_BYTES;
-  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
-
-  int32_t rc = launch_zero_words(stream, hist, (L.total - L.zero_begin) / 4);
-  if (rc != ILGPU_HIP_SUCCESS) return rc;
-
-  {
-    int shift = 0;  // replicas: as many as kHistLdsWords of LDS counters hold
-    while ((1 << (shift + 1)) <= 32 &&
-           ((passes * kRadix) << (shift + 1)) <= kHistLdsWords)
-      ++shift;
-    const size_t lds = (size_t)((passes * kRadix) << shift) * 4;
-    int64_t blocks = div_up(div_up(a.n, Vec16<K>::N), kHistBlock);
-    // Two blocks of 64 KiB of counters are resident per CU: no second round.
-    if (blocks > (int64_t)cus * 2) blocks = (int64_t)cus * 2;
-    if (blocks < 1) blocks = 1;
-    ProfileScope scope(stream, "sort_histogram");
-    hipLaunchKernelGGL((sort_histogram_kernel<K>), dim3((unsigned)blocks),
-                       dim3(kHistBlock), lds, stream, keys_a, a.n, xf, passes,
-                       shift, hist);
-    ILGPU_HIP_CHECK(hipGetLastError());
-  }
-  {
-    ProfileScope scope(stream, "sort_plan");
-    hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(kRadix), 0, stream, hist, excl,
-                       plan, passes, (uint32_t)a.n);
-  }
-  ILGPU_HIP_CHECK(hipGetLastError());
-
-  if (use_large)
-    rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlockLarge>(stream, a, L, base, xf, cus);
-  else
-    rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlock>(stream, a, L, base, xf, cus);
-  if (rc != ILGPU_HIP_SUCCESS) return rc;
-  {
-    int64_t blocks = div_up(a.n, 256);
-    if (blocks > (int64_t)cus * 8) blocks = (int64_t)cus * 8;
-    ProfileScope scope(stream, "sort_finish");
-    hipLaunchKernelGGL((finish_kernel<KEY_BYTES, VALUE_BYTES>),
-                       dim3((unsigned)blocks), dim3(256), 0, stream, keys_a,
-                       keys_b, vals_a, vals_b, a.n, plan, from_index);
-    ILGPU_HIP_CHECK(hipGetLastError());
-  }
-  return ILGPU_HIP_SUCCESS;
-}
-
-template <int KEY_BYTES>
-int32_t launch_value(hipStream_t stream, const SortArgs& a) {
-  switch (a.value_bytes) {
-    case 0: return launch_sized<KEY_BYTES, 0>(stream, a);
-    case 1: return launch_sized<KEY_BYTES, 1>(stream, a);
-    case 2: return launch_sized<KEY_BYTES, 2>(stream, a);
-    case 4: return launch_sized<KEY_BYTES, 4>(stream, a);
-    case 8: return launch_sized<KEY_BYTES, 8>(stream, a);
-    case 16: return launch_sized<KEY_BYTES, 16>(stream, a);
-    default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  }
-}
 
 // ---- strided views ------------------------------------------------------------
 // Stride1D.General with an element stride above one: the view is gathered
@@ -1128,10 +108,10 @@ int32_t copy_strided_bytes(hipStream_t stream, bool gather, int elem_bytes, void
 
 int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
   switch (elem_size(a.key_type)) {
-    case 1: return launch_value<1>(stream, a);
-    case 2: return launch_value<2>(stream, a);
-    case 4: return launch_value<4>(stream, a);
-    case 8: return launch_value<8>(stream, a);
+    case 1: return launch_sort_key_bytes_1(stream, a);
+    case 2: return launch_sort_key_bytes_2(stream, a);
+    case 4: return launch_sort_key_bytes_4(stream, a);
+    case 8: return launch_sort_key_bytes_8(stream, a);
     default: return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   }
 }
@@ -1140,9 +120,9 @@ int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
 
 void set_sort_parameter(int32_t parameter, int32_t value) {
   if (parameter == ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT)
-    g_spin_limit.store(value < 0 ? kDefaultSpinLimit : (uint32_t)value, std::memory_order_relaxed);
+    g_sort_spin_limit.store(value < 0 ? kDefaultSpinLimit : (uint32_t)value, std::memory_order_relaxed);
   else
-    g_large_min_tiles_per_cu.store(value < 0 ? -1 : value, std::memory_order_relaxed);
+    g_sort_large_min_tiles_per_cu.store(value < 0 ? -1 : value, std::memory_order_relaxed);
 }
 
 int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches) {

@@ -1,0 +1,10 @@
+// Radix sort of 2-byte keys: instantiates radix_sort_impl.hpp for every value size.
+#include "radix_sort_impl.hpp"
+
+namespace ilgpu_hip {
+
+int32_t launch_sort_key_bytes_2(hipStream_t stream, const SortArgs& a) {
+  return launch_value<2>(stream, a);
+}
+
+}  // namespace ilgpu_hip
