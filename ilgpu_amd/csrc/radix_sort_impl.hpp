@@ -229,7 +229,7 @@ struct SortPlan {
 };
 
 // ---- histogram of all digit positions ------------------------------------
-template <typename K>
+template <typename K, bool FLOAT_KEYS>
 __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
     const K* __restrict__ keys, int64_t n, KeyXform xf, int passes,
     int replica_shift, uint32_t* __restrict__ global_hist) {
@@ -241,15 +241,17 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
   __syncthreads();
 
   const uint32_t replica = threadIdx.x & ((1u << replica_shift) - 1u);
-  const bool has_term = (xf.reference_term | xf.total_term) != 0;  // float keys
   auto count = [&](K k) {
     K o = (K)(k ^ (K)xf.xor_mask);
-    if (has_term) o ^= key_term(k, xf);
+    if constexpr (FLOAT_KEYS) o ^= key_term(k, xf);
 #pragma unroll
     for (int p = 0; p < (int)sizeof(K); ++p) {
       const uint32_t d = (uint32_t)(o >> (8 * p)) & (kRadix - 1);
       atomicAdd(&s_hist[((p * kRadix + d) << replica_shift) + replica], 1u);
     }
+    // Key by key: with the digits of all keys of a vector extracted first and
+    // their atomics issued in one burst the kernel measured 4 % slower.
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   const uintptr_t addr = reinterpret_cast<uintptr_t>(keys);
@@ -1007,7 +1009,11 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
     if (blocks > (int64_t)cus * 2) blocks = (int64_t)cus * 2;
     if (blocks < 1) blocks = 1;
     ProfileScope scope(stream, "sort_histogram");
-    hipLaunchKernelGGL((sort_histogram_kernel<K>), dim3((unsigned)blocks),
+    auto* histogram_kernel = sort_histogram_kernel<K, false>;
+    if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
+      if ((xf.reference_term | xf.total_term) != 0) histogram_kernel = sort_histogram_kernel<K, true>;
+    }
+    hipLaunchKernelGGL(histogram_kernel, dim3((unsigned)blocks),
                        dim3(kHistBlock), lds, stream, keys_a, a.n, xf, passes,
                        shift, hist);
     ILGPU_HIP_CHECK(hipGetLastError());
