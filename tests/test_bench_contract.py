@@ -1,0 +1,52 @@
+"""bench.py's command-line contract and the provenance of its traffic figures
+(no GPU: nothing here launches a kernel)."""
+import json
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+import bench  # noqa: E402
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode != 0
+    assert "one GPU" in (proc.stdout + proc.stderr)
+
+
+def test_traffic_table_names_sources_that_exist_and_carries_its_commands():
+    with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+        table = json.load(f)
+    assert all("rocprofv3 --pmc" in c and "bench.py" in c for c in table["commands"])
+    assert "radix_sort_u32_uniform_2^28" in table["workloads"]
+    for name, entry in table["workloads"].items():
+        assert os.path.exists(os.path.join(bench.CSRC, entry["source"])), name
+        assert entry["bytes_per_launch"] > 0 and len(entry["sha256"]) == 16, name
+
+
+def test_source_digest_ignores_comments_and_layout_but_not_code(tmp_path, monkeypatch):
+    monkeypatch.setattr(bench, "CSRC", str(tmp_path))
+    (tmp_path / "a.hip").write_text("int f() {\n  return 1;  // one\n}\n")
+    (tmp_path / "b.hip").write_text("// header\n\nint f() {\n      return 1;\n}\n")
+    (tmp_path / "c.hip").write_text("int f() {\n  return 2;\n}\n")
+    assert bench.source_digest("a.hip") == bench.source_digest("b.hip")
+    assert bench.source_digest("a.hip") != bench.source_digest("c.hip")
+
+
+def test_stale_counters_are_not_reported_as_traffic(tmp_path, monkeypatch):
+    # counters read on other code: no figure, and the provenance says why
+    table = {"workloads": {"w": {"bytes_per_launch": 5.0, "source": "a.hip", "sha256": "0" * 16}}}
+    path = tmp_path / "t.json"
+    path.write_text(json.dumps(table))
+    (tmp_path / "a.hip").write_text("int f() { return 1; }\n")
+    monkeypatch.setattr(bench, "CSRC", str(tmp_path))
+    monkeypatch.setattr(bench, "TRAFFIC_FILE", str(path))
+    value, provenance = bench.measured_traffic("w", True)
+    assert value is None and "stale" in provenance
+    table["workloads"]["w"]["sha256"] = bench.source_digest("a.hip")
+    path.write_text(json.dumps(table))
+    value, provenance = bench.measured_traffic("w", True)
+    assert value == 5.0 and "stale" not in provenance
