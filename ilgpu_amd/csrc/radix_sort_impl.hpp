@@ -69,8 +69,14 @@ constexpr int kMaxPasses = 8;
 #ifndef ILGPU_HIP_SORT_ITEMS8
 #define ILGPU_HIP_SORT_ITEMS8 18
 #endif
+#ifndef ILGPU_HIP_SORT_PAIR_ITEMS2
+#define ILGPU_HIP_SORT_PAIR_ITEMS2 16
+#endif
+#ifndef ILGPU_HIP_SORT_PAIR_ITEMS4
+#define ILGPU_HIP_SORT_PAIR_ITEMS4 10
+#endif
 #ifndef ILGPU_HIP_SORT_PAIR_ITEMS3
-#define ILGPU_HIP_SORT_PAIR_ITEMS3 16
+#define ILGPU_HIP_SORT_PAIR_ITEMS3 14
 #endif
 #ifndef ILGPU_HIP_SORT_LOOKBACK
 #define ILGPU_HIP_SORT_LOOKBACK 4
@@ -159,15 +165,21 @@ template <> struct ValueOf<16> { using type = Bytes16; };
 // Keys per thread and tile.  Long tiles pay: the runs they scatter are longer
 // (fewer partial cache lines) and there are fewer tiles to chain.  Keys-only
 // sorts take 36 keys of up to 4 bytes or 18 of 8 bytes per thread: the most
-// that lets two blocks share a compute unit's 160 KiB of LDS.  Values live in
-// registers next to the keys, which caps pairs lower, by the registers one
-// pair takes: 20 items at two (key and value of up to 4 bytes each), 16 at
-// three, 14 at four, 8 with 16-byte values.  (Measured at 12 to 24 items.)
+// that the 160 KiB of LDS of a compute unit stage for sixteen waves.  Values
+// live in registers next to the keys, which caps pairs lower, by the registers
+// one pair takes: at two (key and value of up to 4 bytes each) 16 items with
+// 4-byte values and 20 with shorter ones, 14 at three, 10 at four, 8 with
+// 16-byte values.  (Measured per pass on 2^27 pairs with 1024-thread blocks:
+// u32 + u32 at 16 / 18 / 20 / 24 items 0.470 / 0.486 / 0.486 / 0.972 ms; u64 +
+// u32 at 10 / 12 / 14 / 16 / 18 items 0.714 / 0.681 / 0.667 / 0.702 / 0.691;
+// u64 + u64 at 10 / 12 / 14 items 0.902 / 0.919 / 0.947; u32 + u8 at 16 / 18 /
+// 20 items 0.597 / 0.594 / 0.579.)
 constexpr int items_per_thread(int key_bytes, int value_bytes) {
   if (value_bytes == 0) return key_bytes == 8 ? ILGPU_HIP_SORT_ITEMS8 : ILGPU_HIP_SORT_ITEMS;
   if (value_bytes == 16) return 8;
   const int registers = (key_bytes == 8 ? 2 : 1) + (value_bytes == 8 ? 2 : 1);
-  return registers == 2 ? 20 : registers == 3 ? ILGPU_HIP_SORT_PAIR_ITEMS3 : 14;
+  if (registers == 2) return value_bytes <= 2 ? 20 : ILGPU_HIP_SORT_PAIR_ITEMS2;
+  return registers == 3 ? ILGPU_HIP_SORT_PAIR_ITEMS3 : ILGPU_HIP_SORT_PAIR_ITEMS4;
 }
 constexpr int tile_keys(int key_bytes, int value_bytes, int block) {
   return block * items_per_thread(key_bytes, value_bytes);
