@@ -391,8 +391,19 @@ template <int KEY_BYTES, int VALUE_BYTES, int BLOCK> struct SortTile {
   static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES, BLOCK);
   static constexpr int kSubTileKeys = kSubLanes * kItems;
   static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
-  static constexpr int kStageBytes =
+  // The values of a tile go through the same LDS bytes after the keys, all at
+  // once when they fit (72 KiB per 512 threads: two such blocks or one of 1024
+  // threads share a compute unit's LDS), else in rounds.
+#ifndef ILGPU_HIP_SORT_VALUE_STAGE
+#define ILGPU_HIP_SORT_VALUE_STAGE 1
+#endif
+  static constexpr int kValueStageLimit = ILGPU_HIP_SORT_VALUE_STAGE ? (BLOCK / 512) * 72 * 1024 : 0;
+  static constexpr int kValueStageBytes =
+      kTile * VALUE_BYTES <= kValueStageLimit ? kTile * VALUE_BYTES : 0;
+  static constexpr int kKeyOrCounterBytes =
       kCounterBytes > kKeyStageBytes ? kCounterBytes : kKeyStageBytes;
+  static constexpr int kStageBytes =
+      kValueStageBytes > kKeyOrCounterBytes ? kValueStageBytes : kKeyOrCounterBytes;
 };
 
 template <int KEY_BYTES, int ITEMS, bool FULL>
