@@ -319,6 +319,7 @@ def selftest_lds_atomic_order(rows: int = 256, *, stream=None) -> int:
 
 SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0
 SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1
+SORT_PARAM_ONE_TILE_KERNEL = 2
 
 
 def sort_set_parameter(parameter: int, value: int) -> None:

@@ -8,6 +8,7 @@ namespace ilgpu_hip {
 
 std::atomic<uint32_t> g_sort_spin_limit{kDefaultSpinLimit};
 std::atomic<int32_t> g_sort_large_min_tiles_per_cu{-1};
+std::atomic<int32_t> g_sort_small_kernel{1};
 
 // radix_sort_k<bytes>.hip
 int32_t launch_sort_key_bytes_1(hipStream_t stream, const SortArgs& a);
@@ -121,8 +122,10 @@ int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
 void set_sort_parameter(int32_t parameter, int32_t value) {
   if (parameter == ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT)
     g_sort_spin_limit.store(value < 0 ? kDefaultSpinLimit : (uint32_t)value, std::memory_order_relaxed);
-  else
+  else if (parameter == ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU)
     g_sort_large_min_tiles_per_cu.store(value < 0 ? -1 : value, std::memory_order_relaxed);
+  else
+    g_sort_small_kernel.store(value == 0 ? 0 : 1, std::memory_order_relaxed);
 }
 
 int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches) {

@@ -52,6 +52,7 @@ namespace ilgpu_hip {
 // radix_sort.hip.
 extern std::atomic<uint32_t> g_sort_spin_limit;
 extern std::atomic<int32_t> g_sort_large_min_tiles_per_cu;  // negative: the defaults
+extern std::atomic<int32_t> g_sort_small_kernel;            // 0: one-tile inputs take the passes too
 
 namespace {
 
@@ -854,6 +855,152 @@ void onesweep_kernel(
   }
 }
 
+// ---- inputs of one tile ---------------------------------------------------------
+// A sort of at most one 512-thread tile runs as one block and one launch: the
+// keys (and values) stay in registers, every pass ranks them like a pass above,
+// moves them through LDS into digit order and takes them back in memory order
+// (lane l of wave w holds positions w*64*I + j*64 + l again), and the last pass
+// is followed by one coalesced write.  No histogram, plan, tickets, look-back
+// or temp memory; a pass whose digit is the same for every key simply leaves
+// the order as it is.
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS>
+__global__ __launch_bounds__(kSortBlock, ILGPU_HIP_SORT_WAVES_PER_EU)
+void small_sort_kernel(typename KeyOf<KEY_BYTES>::type* keys,
+                       typename ValueOf<VALUE_BYTES>::type* vals, int n, KeyXform xf,
+                       int values_from_index) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  using Val = typename ValueOf<VALUE_BYTES>::type;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, kSortBlock>;
+  constexpr int kItems = TileCfg::kItems;
+  constexpr int kSubTiles = TileCfg::kSubTiles;
+  constexpr bool kPairs = VALUE_BYTES > 0;
+  static_assert(!kPairs || TileCfg::kTile * VALUE_BYTES <= TileCfg::kStageBytes,
+                "the values of a tile are staged at once");
+
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[TileCfg::kStageBytes];
+  __shared__ uint32_t s_scan[kRadix / kWaveSize];
+  uint32_t* s_counter = reinterpret_cast<uint32_t*>(s_stage);
+  K* s_keys = reinterpret_cast<K*>(s_stage);
+  Val* s_vals = reinterpret_cast<Val*>(s_stage);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int wave = tid / kWaveSize;
+  const int first_local = wave * TileCfg::kSubTileKeys + lane;
+  uint32_t* my_counters = s_counter + wave * kRadix;
+
+  K key[kItems];
+  Val val[kPairs ? kItems : 1];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const int local = first_local + j * kSubLanes;
+    key[j] = 0;
+    if (local < n) {
+      key[j] = keys[local];
+      if constexpr (FLOAT_KEYS) key[j] = ordered_bits(key[j], xf);
+      if constexpr (kPairs) {
+        if (values_from_index) {
+          if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)local;
+          else if constexpr (VALUE_BYTES == 8) val[j] = (Val)(uint64_t)local;
+        } else {
+          val[j] = vals[local];
+        }
+      }
+    }
+  }
+
+#pragma unroll 1
+  for (int pass = 0; pass < KEY_BYTES; ++pass) {
+    const int shift = pass * 8;
+    // Positions past the end take digit 255 and come last in memory order, so
+    // they stay behind every key through every pass.
+    auto item_digit = [&](int j) -> uint32_t {
+      if (first_local + j * kSubLanes >= n) return (uint32_t)(kRadix - 1);
+      if constexpr (FLOAT_KEYS) return (uint32_t)(key[j] >> shift) & (kRadix - 1);
+      else return (uint32_t)((K)(key[j] ^ (K)xf.xor_mask) >> shift) & (kRadix - 1);
+    };
+    __syncthreads();  // the stage of the previous pass has been read
+    for (int i = tid; i < TileCfg::kCounterWords; i += kSortBlock) s_counter[i] = 0u;
+    __syncthreads();
+
+    uint32_t packed[kItems / 2];  // rank in the sub-tile, then position in the tile
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const uint32_t d = item_digit(j);
+      // a row that is all one digit: lane 0 adds for the row (see sort_tile)
+      const uint32_t row_digit = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+      const bool whole_row = __ballot(d == row_digit) == ~0ull;
+      uint32_t rank = 0;
+      if (!whole_row || lane == 0)
+        rank = __hip_atomic_fetch_add(my_counters + d, whole_row ? (uint32_t)kSubLanes : 1u,
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (whole_row) rank = (uint32_t)__builtin_amdgcn_readfirstlane((int)rank) + (uint32_t)lane;
+      if (j % 2 == 0) packed[j / 2] = rank;
+      else packed[j / 2] |= rank << 16;
+    }
+    __syncthreads();
+
+    // One thread per digit: totals over the sub-tiles, exclusive scan over the
+    // digits, then the tile position of the first key of every (sub-tile, digit).
+    uint32_t count = 0, inc = 0;
+    if (tid < kRadix) {
+#pragma unroll
+      for (int s = 0; s < kSubTiles; ++s) count += s_counter[s * kRadix + tid];
+      inc = count;
+#pragma unroll
+      for (int s = 1; s < kWaveSize; s <<= 1) {
+        const uint32_t o = shfl_up(inc, s);
+        if (lane >= s) inc += o;
+      }
+      if (lane == kWaveSize - 1) s_scan[wave] = inc;
+    }
+    __syncthreads();
+    if (tid < kRadix) {
+      uint32_t run = inc - count;
+      for (int w = 0; w < wave; ++w) run += s_scan[w];
+#pragma unroll
+      for (int s = 0; s < kSubTiles; ++s) {
+        const uint32_t t = s_counter[s * kRadix + tid];
+        s_counter[s * kRadix + tid] = run;
+        run += t;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kItems; j += 2) {
+      const uint32_t p0 = my_counters[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
+      const uint32_t p1 = my_counters[item_digit(j + 1)] + (packed[j / 2] >> 16);
+      packed[j / 2] = p0 | (p1 << 16);
+    }
+    __syncthreads();  // the run starts have been read; the same bytes stage the keys
+#pragma unroll
+    for (int j = 0; j < kItems; ++j)
+      s_keys[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = key[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) key[j] = s_keys[first_local + j * kSubLanes];
+    if constexpr (kPairs) {
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < kItems; ++j)
+        s_vals[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = val[j];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < kItems; ++j) val[j] = s_vals[first_local + j * kSubLanes];
+    }
+  }
+
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const int local = first_local + j * kSubLanes;
+    if (local < n) {
+      if constexpr (FLOAT_KEYS) keys[local] = raw_bits(key[j], xf);
+      else keys[local] = key[j];
+      if constexpr (kPairs) vals[local] = val[j];
+    }
+  }
+}
+
 // ---- finish ----------------------------------------------------------------
 template <int KEY_BYTES, int VALUE_BYTES>
 __global__ __launch_bounds__(256) void finish_kernel(
@@ -997,6 +1144,22 @@ template <int KEY_BYTES, int VALUE_BYTES>
 int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
+  if (a.n <= (int64_t)tile_keys(KEY_BYTES, VALUE_BYTES, kSortBlock) &&
+      g_sort_small_kernel.load(std::memory_order_relaxed) != 0) {
+    // one tile: one block, one launch, no temp
+    const KeyXform xf = make_xform(a.key_type, a.flags);
+    auto* kernel = small_sort_kernel<KEY_BYTES, VALUE_BYTES, false>;
+    if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
+      if ((xf.reference_term | xf.total_term) != 0)
+        kernel = small_sort_kernel<KEY_BYTES, VALUE_BYTES, true>;
+    }
+    ProfileScope scope(stream, "sort_small");
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(kSortBlock), 0, stream, static_cast<K*>(a.keys),
+                       static_cast<Val*>(a.values), (int)a.n, xf,
+                       a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0);
+    ILGPU_HIP_CHECK(hipGetLastError());
+    return ILGPU_HIP_SUCCESS;
+  }
   const int cus = device_cu_count();
   int64_t min_tiles_per_cu = g_sort_large_min_tiles_per_cu.load(std::memory_order_relaxed);
   if (min_tiles_per_cu < 0)

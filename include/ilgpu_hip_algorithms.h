@@ -205,10 +205,15 @@ int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
  *     tiles per compute unit are sorted with 1024-thread blocks (longer runs
  *     per digit), smaller ones with 512-thread blocks (more blocks for fewer
  *     keys).  Default 10 for keys, 2 for pairs; 0 = always the large block,
- *     INT32_MAX = never. */
+ *     INT32_MAX = never.
+ *   ONE_TILE_KERNEL  inputs of at most one 512-thread tile (18432 keys of up
+ *     to 4 bytes, fewer for wider keys and for pairs) are sorted by one block
+ *     in one launch, without temp memory.  Default 1; 0 sends them through
+ *     the passes like longer inputs. */
 enum {
   ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0,
-  ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1
+  ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1,
+  ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL = 2
 };
 int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value);
 

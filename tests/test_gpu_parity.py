@@ -694,6 +694,71 @@ def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
 
 
 @pytest.fixture
+def no_one_tile_kernel():
+    """Inputs of one tile go through histogram, plan and passes like longer ones
+    (by default one block sorts them in one launch)."""
+    capi.sort_set_parameter(capi.SORT_PARAM_ONE_TILE_KERNEL, 0)
+    yield
+    capi.sort_set_parameter(capi.SORT_PARAM_ONE_TILE_KERNEL, 1)
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+def test_sort_of_one_tile_through_the_passes_matches_oracle(no_one_tile_kernel, dtype):
+    kinds = np.dtype(dtype).kind
+    for n in [1, 2, 63, 64, 65, 1027, 4097, 9216, 18431, 18432]:
+        note("one tile through the passes", np.dtype(dtype).name, n)
+        keys = random_float_bits(dtype, n, seed=n) if kinds == "f" else random_ints(dtype, n, seed=n)
+        for descending in (False, True):
+            assert bits_equal(gpu_sort(keys, descending=descending),
+                              O.radix_sort(keys, descending=descending)), (n, descending)
+    keys = (random_ints(np.int32, 5000, seed=3, lo=-40, hi=40)).astype(dtype)
+    values = np.arange(keys.size, dtype=np.uint32)
+    k, v = gpu_sort_pairs(keys, values)
+    ek, ev = O.radix_sort_pairs(keys, values)
+    assert bits_equal(k, ek) and np.array_equal(v, ev)
+
+
+@pytest.mark.parametrize("key_dtype,value_dtype", [
+    (np.uint32, np.uint32), (np.uint64, np.uint32), (np.uint32, np.uint64), (np.int64, np.float64),
+    (np.uint8, np.uint8), (np.int16, np.uint16), (np.float32, np.int32), (np.float16, np.uint64),
+    (np.float64, np.uint8)])
+def test_sort_pairs_of_one_tile_by_one_block(key_dtype, value_dtype):
+    # sizes up to the tile of every pair type (4096 pairs with 16-byte values,
+    # 5120 to 10240 otherwise) and just beyond, where the passes take over
+    for n in [1, 2, 64, 65, 1000, 4095, 4096, 4097, 5120, 5121, 7168, 7169, 8192, 8193, 10240,
+              10241]:
+        note("one-tile pairs", np.dtype(key_dtype).name, np.dtype(value_dtype).name, n)
+        keys = (random_ints(np.int32, n, seed=n, lo=-40, hi=40)).astype(key_dtype)
+        values = np.arange(n).astype(value_dtype)
+        for descending in (False, True):
+            k, v = gpu_sort_pairs(keys, values, descending=descending)
+            ek, ev = O.radix_sort_pairs(keys, values, descending=descending)
+            assert bits_equal(k, ek) and bits_equal(v, ev), (n, descending)
+    n = 4000
+    keys = random_ints(np.uint32, n, seed=5, lo=0, hi=300)
+    order = np.argsort(keys, kind="stable")
+    values = np.zeros((n, 2), dtype=np.uint64)
+    values[:, 0] = np.arange(n)
+    values[:, 1] = ~np.arange(n, dtype=np.uint64)
+    dk = D.from_numpy(keys)
+    dv = D(n, np.dtype([("a", np.uint64), ("b", np.uint64)]),
+           _bytes=D.from_numpy(values.reshape(-1)).bytes)
+    temp = capi.temp_buffer(capi.radix_sort_temp_bytes(n, np.uint32, 16))
+    capi.check(capi.lib().ilgpu_hip_radix_sort_pairs(
+        None, dk.ptr, 1, dv.ptr, 1, n, capi.U32, 16, 0, capi.VALUES_FROM_VIEW,
+        temp.ptr, temp.nbytes))
+    sync()
+    assert np.array_equal(dk.numpy(), keys[order])
+    assert np.array_equal(dv.bytes.cpu().numpy().view(np.uint64).reshape(n, 2), values[order])
+    dk2, dv2 = D.from_numpy(keys), D.zeros(n, np.uint64)
+    capi.radix_sort_pairs(dk2, dv2, values_from_index=True, descending=True)
+    sync()
+    order_desc = np.argsort(~keys, kind="stable")
+    assert np.array_equal(dk2.numpy(), keys[order_desc])
+    assert np.array_equal(dv2.numpy(), order_desc.astype(np.uint64))
+
+
+@pytest.fixture
 def large_sort_blocks():
     """Sorts of any size take the 1024-thread kernels (by default only inputs of
     tens of millions of keys do)."""
