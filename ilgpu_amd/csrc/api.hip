@@ -390,7 +390,8 @@ int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void* in,
   const int eb = elem_size(in_type);
   if (eb < 0 || in_type == ILGPU_HIP_F16) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (bin_type != ILGPU_HIP_I32 && bin_type != ILGPU_HIP_U32 &&
-      bin_type != ILGPU_HIP_I64 && bin_type != ILGPU_HIP_U64)
+      bin_type != ILGPU_HIP_I64 && bin_type != ILGPU_HIP_U64 &&
+      bin_type != ILGPU_HIP_F32 && bin_type != ILGPU_HIP_F64)
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (locator != ILGPU_HIP_LOCATOR_IDENTITY &&
       locator != ILGPU_HIP_LOCATOR_MODULO)

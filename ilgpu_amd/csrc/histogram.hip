@@ -114,6 +114,78 @@ __device__ __forceinline__ bool add_to_bin(void* bins, int64_t b, uint32_t c,
   }
 }
 
+// ---- floating-point bins ------------------------------------------------------
+// The reference adds 1.0 to a float or double bin once per element, each
+// addition rounded in the bin's precision (Atomic.Add(ref target, 1),
+// HistogramOperations.tt:36-40), so a float bin stops growing at 2^24.  Every
+// increment is the same function x -> fl(x + 1), so the value of a bin after c
+// of them does not depend on their order, and add_ones gives exactly that
+// value without c additions: inside a binade whose spacing is at most one,
+// steps of one are exact (x, 1 and x + 1 are multiples of the spacing), so
+// whole runs of steps up to the top of the binade (or, for negative values,
+// down to magnitude below one) are taken at once; the steps that can round —
+// into a coarser binade, across zero, beyond 2^24 or 2^53 — are single
+// additions in hardware.
+template <typename F>
+__device__ __forceinline__ F add_ones(F x, uint32_t c) {
+  constexpr int kDigits = sizeof(F) == 4 ? 24 : 53;
+  const F limit = (F)(1ull << kDigits);
+  if (x != x) return x;  // NaN stays NaN
+  while (c > 0) {
+    const F y = x + (F)1;
+    if (y == x) return x;  // stuck: the spacing has outgrown one (or x is infinite)
+    uint32_t k = 1;
+    F next = y;
+    const F ax = x < (F)0 ? -x : x;
+    if (ax >= (F)1 && ax < limit) {
+      uint64_t whole;
+      if (x > (F)0) {
+        int e;
+        if constexpr (sizeof(F) == 4) (void)frexpf(x, &e);
+        else (void)frexp(x, &e);
+        F top;  // 2^e: the first value of the next binade, above x
+        if constexpr (sizeof(F) == 4) top = ldexpf(1.0f, e);
+        else top = ldexp(1.0, e);
+        whole = (uint64_t)(top - x);  // steps that end at or below it
+      } else {
+        whole = (uint64_t)ax;         // steps that end at or below zero
+      }
+      if (whole >= 1) {
+        k = whole < (uint64_t)c ? (uint32_t)whole : c;
+        next = x + (F)k;  // exact
+      }
+    }
+    x = next;
+    c -= k;
+  }
+  return x;
+}
+
+// Adds c ones to the floating-point bin b; returns whether an increment found
+// the bin at MaxValue (only a bin that holds MaxValue already: it is not
+// reachable by steps of one).
+template <typename F, typename U>
+__device__ __forceinline__ bool add_to_fp_bin(void* bins, int64_t b, uint32_t c,
+                                              bool checked) {
+  U* p = static_cast<U*>(bins) + b;
+  U old = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    F x;
+    __builtin_memcpy(&x, &old, sizeof(F));
+    const F y = add_ones<F>(x, c);
+    U desired;
+    __builtin_memcpy(&desired, &y, sizeof(F));
+    if (desired == old) break;  // nothing to store
+    if (__hip_atomic_compare_exchange_strong(p, &old, desired, __ATOMIC_RELAXED,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      break;
+  }
+  F before;
+  __builtin_memcpy(&before, &old, sizeof(F));
+  const F max_value = sizeof(F) == 4 ? (F)3.402823466e+38f : (F)1.7976931348623157e+308;
+  return checked && before == max_value;
+}
+
 __device__ __forceinline__ bool add_to_bin_dyn(int bin_type, void* bins,
                                                int64_t b, uint32_t c,
                                                bool checked) {
@@ -121,6 +193,8 @@ __device__ __forceinline__ bool add_to_bin_dyn(int bin_type, void* bins,
     case ILGPU_HIP_I32: return add_to_bin<int32_t>(bins, b, c, checked);
     case ILGPU_HIP_U32: return add_to_bin<uint32_t>(bins, b, c, checked);
     case ILGPU_HIP_I64: return add_to_bin<int64_t>(bins, b, c, checked);
+    case ILGPU_HIP_F32: return add_to_fp_bin<float, uint32_t>(bins, b, c, checked);
+    case ILGPU_HIP_F64: return add_to_fp_bin<double, uint64_t>(bins, b, c, checked);
     default: return add_to_bin<uint64_t>(bins, b, c, checked);
   }
 }

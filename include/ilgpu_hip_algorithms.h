@@ -276,9 +276,14 @@ int32_t ilgpu_hip_reduce(ilgpu_hip_stream_t stream, const void *in,
  * Replaces: Histogram / HistogramUnchecked delegates and launchers
  * (HistogramExtensions.cs:35-59, 293-508; HistogramLaunchers.tt:52-101).
  * bins[locator(v)] += 1 for every input element; bins are ACCUMULATED into,
- * never cleared.  bin_type in {I32, I64, U32, U64}.  If `overflow` is not
- * NULL, overflow[0] |= 1 when some bin's count passed the bin type's MaxValue
- * (HistogramOperations.tt:36-40); NULL selects the unchecked variant.
+ * never cleared.  bin_type in {I32, I64, U32, U64, F32, F64}: the reference's
+ * AtomicNumericTypes.  A floating-point bin receives its additions of 1.0 one
+ * by one in its own precision, as Atomic.Add does, so a float bin stops
+ * growing at 2^24 (16777216 + 1 rounds back to 16777216); the result is
+ * computed exactly and does not depend on the order of the elements.  If
+ * `overflow` is not NULL, overflow[0] |= 1 when some bin's count passed the
+ * bin type's MaxValue (an increment found the bin holding MaxValue,
+ * HistogramOperations.tt:36-40); NULL selects the unchecked variant.
  * in_type: any ilgpu_hip_type except F16.
  */
 int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void *in,

@@ -10,6 +10,7 @@
  */
 #include "ilgpu_cpu_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -540,6 +541,29 @@ DEFINE_HIST(i64, int64_t, uint64_t, INT64_MAX)
 DEFINE_HIST(u32, uint32_t, uint32_t, UINT32_MAX)
 DEFINE_HIST(u64, uint64_t, uint64_t, UINT64_MAX)
 
+/* Floating-point bins (HistogramLaunchers.tt:25 over AtomicNumericTypes, which
+ * include float and double): Atomic.Add(ref target, 1) adds 1.0 in the bin's
+ * own precision, one rounding per element (HistogramOperations.tt:36-40); a
+ * float bin therefore stops growing at 2^24.  volatile keeps every addition in
+ * the bin's precision. */
+#define DEFINE_HIST_FP(NAME, T, TMAX)                                          \
+  static int hist_##NAME(int in_type, int locator, const void *in, int64_t n,  \
+                         T *bins, int64_t num_bins, int32_t *overflow) {       \
+    int did = 0;                                                               \
+    for (int64_t i = 0; i < n; ++i) {                                          \
+      int64_t b = locate_bin(in_type, locator, in, i, num_bins);               \
+      if (b < 0 || b >= num_bins) return -2;                                   \
+      volatile T old = bins[b];                                                \
+      volatile T next = old + (T)1;                                            \
+      bins[b] = next;                                                          \
+      did |= old == (TMAX);                                                    \
+    }                                                                          \
+    if (overflow) *overflow |= did ? 1 : 0;                                    \
+    return 0;                                                                  \
+  }
+DEFINE_HIST_FP(f32, float, FLT_MAX)
+DEFINE_HIST_FP(f64, double, DBL_MAX)
+
 int oracle_histogram(int in_type, int bin_type, int locator, const void *in,
                      int64_t n, void *bins, int64_t num_bins,
                      int32_t *overflow) {
@@ -551,6 +575,8 @@ int oracle_histogram(int in_type, int bin_type, int locator, const void *in,
     case ORACLE_I64: return hist_i64(in_type, locator, in, n, bins, num_bins, overflow);
     case ORACLE_U32: return hist_u32(in_type, locator, in, n, bins, num_bins, overflow);
     case ORACLE_U64: return hist_u64(in_type, locator, in, n, bins, num_bins, overflow);
+    case ORACLE_F32: return hist_f32(in_type, locator, in, n, bins, num_bins, overflow);
+    case ORACLE_F64: return hist_f64(in_type, locator, in, n, bins, num_bins, overflow);
     default: return -1;
   }
 }

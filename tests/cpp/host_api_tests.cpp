@@ -524,6 +524,39 @@ static void ReduceOnTwoStreams(Accelerator& accl) {
   CHECK(futureB.get() == sumB);
 }
 
+// Floating-point bins (the launchers exist for every AtomicNumericType,
+// HistogramLaunchers.tt:25-34): counts below 2^24 are exact in a float bin, a bin
+// near 2^24 stops there, and a bin that holds MaxValue reports overflow
+// (HistogramOperations.tt:36-40).
+template <typename T, typename TBin> void HistogramFloatBinTests(Accelerator& accl) {
+  using Modulo = HistogramOperations::ModuloBinOperation;
+  const int length = 1024, numBins = 64;
+  std::vector<T> input((size_t)length);
+  for (int i = 0; i < length; ++i) input[i] = (T)(i + 1);
+  std::vector<TBin> start((size_t)numBins), expected((size_t)numBins);
+  for (int b = 0; b < numBins; ++b) {
+    start[b] = (TBin)(0.5 * b);
+    expected[b] = (TBin)(0.5 * b + length / numBins);
+  }
+  start[3] = (TBin)16777210.0;  // 16 more: a float bin stops at 2^24
+  expected[3] = sizeof(TBin) == 4 ? (TBin)16777216.0 : (TBin)16777226.0;
+  auto dIn = accl.Allocate1D<T>(input);
+  auto hist = accl.Allocate1D<TBin>(start);
+  auto overflow = accl.Allocate1D<int32_t>(1);
+  overflow->MemSetToZero();
+  Histogram<T, Stride1D::Dense, Modulo, TBin>(accl, accl.DefaultStream(), dIn->View(),
+                                              hist->View(), overflow->View());
+  accl.Synchronize();
+  CHECK(Verify(hist->GetAsArray1D(), expected));
+  CHECK(overflow->GetAsArray1D()[0] == 0);
+  auto full = accl.Allocate1D<TBin>(std::vector<TBin>{std::numeric_limits<TBin>::max()});
+  Histogram<T, Stride1D::Dense, Modulo, TBin>(accl, accl.DefaultStream(), dIn->View(),
+                                              full->View(), overflow->View());
+  accl.Synchronize();
+  CHECK(full->GetAsArray1D()[0] == std::numeric_limits<TBin>::max());
+  CHECK(overflow->GetAsArray1D()[0] == 1);
+}
+
 // ---- HistogramTests -----------------------------------------------------------
 template <typename T, typename TBin> void HistogramTests(Accelerator& accl) {
   using Modulo = HistogramOperations::ModuloBinOperation;
@@ -634,6 +667,8 @@ int main(int argc, char** argv) {
     RUN((HistogramTests<int64_t, int64_t>(accl)));
     RUN((HistogramTests<float, uint64_t>(accl)));
     RUN((HistogramTests<int16_t, int32_t>(accl)));
+    RUN((HistogramFloatBinTests<int32_t, float>(accl)));
+    RUN((HistogramFloatBinTests<float, double>(accl)));
     RUN(UniqueTests<int32_t>(accl));
     RUN(UniqueTests<uint8_t>(accl));
     RUN(UniqueTests<int64_t>(accl));

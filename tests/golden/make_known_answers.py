@@ -170,6 +170,28 @@ def main():
     cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "int32", "locator": "modulo",
                   "input": [0] * 32, "bins_before": [imax - 1, 0],
                   "expected": [wrap(imax - 1 + 32, 32, True), 0], "expected_overflow": 1})
+    # Floating-point bins (HistogramLaunchers.tt over AtomicNumericTypes): 1.0 is added
+    # per element in the bin's precision.  Worked by hand: integers below 2^24 (float) are
+    # exact, so 1..1024 by v % 64 adds 16 to every bin whatever it held; 16777214 + 5
+    # steps is 16777215, 16777216 and then 16777216 + 1 = 16777217, which lies halfway
+    # between 16777216 and 16777218 and rounds to the even mantissa, 16777216: stuck;
+    # -2.5 + 4 steps is 1.5; 0.5 + 3 steps is 3.5; a bin at float.MaxValue stays there and
+    # reports overflow; double bins hold 2^24 + 5 exactly.
+    for bin_dtype in ("float32", "float64"):
+        cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": bin_dtype,
+                      "locator": "modulo", "input": list(range(1, 1025)),
+                      "bins_before": [float(i) / 2 for i in range(64)],
+                      "expected": [float(i) / 2 + 16 for i in range(64)], "expected_overflow": 0})
+    cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "float32", "locator": "modulo",
+                  "input": [0] * 5 + [1] * 4 + [2] * 3, "bins_before": [16777214.0, -2.5, 0.5, 7.0],
+                  "expected": [16777216.0, 1.5, 3.5, 7.0], "expected_overflow": 0})
+    cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "float64", "locator": "modulo",
+                  "input": [0] * 7, "bins_before": [16777214.0, 0.25],
+                  "expected": [16777221.0, 0.25], "expected_overflow": 0})
+    fmax = (2 - 2 ** -23) * 2.0 ** 127  # float.MaxValue, exact in a Python float
+    cases.append({"op": "histogram", "dtype": "int32", "bin_dtype": "float32", "locator": "modulo",
+                  "input": [0, 1], "bins_before": [fmax, 0.0], "expected": [fmax, 1.0],
+                  "expected_overflow": 1})
     # transform
     for n in SIZES:
         cases.append({"op": "transform", "dtype": "int32", "target_dtype": "int32",

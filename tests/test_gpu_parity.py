@@ -295,6 +295,51 @@ def test_histogram_identity_ignores_out_of_range_and_unchecked_variant():
     assert ov == 1
 
 
+@pytest.mark.parametrize("bin_dtype", [np.float32, np.float64])
+def test_histogram_floating_point_bins_take_their_ones_in_bin_precision(bin_dtype):
+    # HistogramLaunchers.tt over AtomicNumericTypes: float and double bins get
+    # 1.0 added per element, rounded in the bin's precision each time, so a
+    # float bin stops at 2^24.  The oracle adds serially; the library computes
+    # the same value without the serial additions.
+    rng = np.random.default_rng(21)
+    fmax = np.finfo(bin_dtype).max
+    assorted = np.array([0.0, -0.0, 0.5, 0.1, -0.3, -2.5, 1.5, 3.999, 16777210.0, 16777215.0,
+                         16777216.0, 16777218.0, -16777218.0, -16777220.0, -33554434.0,
+                         8388607.5, -8388607.5, 1e-30, 1e10, -1e10, np.inf, -np.inf, fmax,
+                         -40000.25, 2.0 ** 23 - 0.5, 65535.0], dtype=bin_dtype)
+    # few bins (counters in LDS, one flush per block and bin)
+    values = rng.integers(0, assorted.size, 300000).astype(np.int32)
+    got, ov = gpu_histogram(values, assorted.copy(), capi.LOCATOR_IDENTITY)
+    want, want_ov = O.histogram(values, assorted.copy())
+    assert bits_equal(got, want)
+    assert ov == want_ov == 1            # a bin held MaxValue
+    # bins that saturate on the way: 2^24 is reached after 100000 of 250000 samples
+    start = np.array([2.0 ** 24 - 100000, 5.0, -7.5, 2.0 ** 24 - 3], dtype=bin_dtype)
+    values = (np.arange(1000000) % 4).astype(np.uint8)
+    got, ov = gpu_histogram(values, start.copy(), capi.LOCATOR_IDENTITY)
+    want, want_ov = O.histogram(values, start.copy())
+    assert bits_equal(got, want) and ov == want_ov == 0
+    if bin_dtype == np.float32:
+        assert got[0] == 2.0 ** 24 and got[3] == 2.0 ** 24 and got[1] == 250005.0
+    else:
+        assert got[0] == 2.0 ** 24 + 150000 and got[1] == 250005.0
+    # many bins (global atomics per element), NaN bins stay NaN, unchecked variant
+    nbins = 20000
+    before = (rng.integers(-50, 50, nbins) * 0.25).astype(bin_dtype)
+    before[7] = np.nan
+    values = rng.integers(0, nbins, 150000).astype(np.int32)
+    got, _ = gpu_histogram(values, before.copy(), capi.LOCATOR_IDENTITY, checked=False)
+    want, _ = O.histogram(values, before.copy())
+    assert np.isnan(got[7]) and np.isnan(want[7])
+    got[7] = want[7] = 0
+    assert bits_equal(got, want)
+    # modulo locator and float input
+    samples = rng.normal(0, 300, 50000).astype(np.float32)
+    got, ov = gpu_histogram(samples, np.zeros(64, dtype=bin_dtype), capi.LOCATOR_MODULO)
+    want, want_ov = O.histogram(samples, np.zeros(64, dtype=bin_dtype), O.LOCATOR_MODULO)
+    assert bits_equal(got, want) and ov == want_ov == 0
+
+
 # --------------------------------------------------------------- radix sort
 def gpu_sort(keys, **kw):
     d = D.from_numpy(keys)

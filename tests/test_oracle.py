@@ -509,3 +509,27 @@ def test_transform_float_semantics():
         O.transform(x, np.int32)
     with pytest.raises(ValueError):
         O.transform(x, np.float64, O.TRANSFORM_BIT_COMPLEMENT)
+
+
+def test_histogram_float_bins_add_one_per_element_and_saturate():
+    # HistogramLaunchers.tt over AtomicNumericTypes (float, double): Atomic.Add(ref
+    # bin, 1) per element in the bin's precision; worked by hand: 16777214 -> 15, 16
+    # and then 16777216 + 1 rounds back to 16777216 (tie to the even mantissa).
+    zeros = np.zeros(5, dtype=np.int32)
+    b, ov = O.histogram(zeros, np.array([16777214.0, 0.5], dtype=np.float32))
+    assert b.tolist() == [16777216.0, 0.5] and ov == 0
+    b, ov = O.histogram(zeros, np.array([16777214.0, 0.5], dtype=np.float64))
+    assert b.tolist() == [16777219.0, 0.5] and ov == 0
+    b, ov = O.histogram(np.array([1, 1, 1, 0], dtype=np.uint8), np.array([-2.5, 0.5], dtype=np.float32))
+    assert b.tolist() == [-1.5, 3.5] and ov == 0
+    # -(2^24 + 2) has an odd mantissa: + 1 is a tie that rounds to -2^24, then steps are exact
+    b, _ = O.histogram(np.zeros(3, dtype=np.int32), np.array([-16777218.0], dtype=np.float32))
+    assert b.tolist() == [-16777214.0]
+    # -(2^24 + 4) has an even one: stuck
+    b, _ = O.histogram(np.zeros(3, dtype=np.int32), np.array([-16777220.0], dtype=np.float32))
+    assert b.tolist() == [-16777220.0]
+    fmax = np.finfo(np.float32).max
+    b, ov = O.histogram(np.zeros(2, dtype=np.int32), np.array([fmax], dtype=np.float32))
+    assert b[0] == fmax and ov == 1
+    b, ov = O.histogram(np.zeros(2, dtype=np.int32), np.array([np.inf], dtype=np.float32))
+    assert b[0] == np.inf and ov == 0
