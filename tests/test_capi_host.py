@@ -155,7 +155,9 @@ def test_histogram_argument_validation():
     assert call(nb=0) == capi.ERROR_NULL_VIEW
     assert call(n=1 << 31) == capi.ERROR_NOT_SUPPORTED
     assert call(t=capi.F16) == capi.ERROR_NOT_SUPPORTED
-    assert call(bt=capi.F32) == capi.ERROR_NOT_SUPPORTED
+    # bins: the six AtomicNumericTypes; Half, 8- and 16-bit bins do not exist
+    assert call(bt=capi.F16) == capi.ERROR_NOT_SUPPORTED
+    assert call(bt=capi.U16) == capi.ERROR_NOT_SUPPORTED
     assert call(loc=9) == capi.ERROR_NOT_SUPPORTED
     assert call(stride=0) == capi.ERROR_OUT_OF_RANGE
 
