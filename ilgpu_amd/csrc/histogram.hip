@@ -167,6 +167,15 @@ __device__ __forceinline__ F add_ones(F x, uint32_t c) {
 template <typename F, typename U>
 __device__ __forceinline__ bool add_to_fp_bin(void* bins, int64_t b, uint32_t c,
                                               bool checked) {
+  const F max_value = sizeof(F) == 4 ? (F)3.402823466e+38f : (F)1.7976931348623157e+308;
+  if (c == 1u) {
+    // One element: the hardware's floating-point add in L2 is the reference's
+    // operation itself (one addition of 1.0, rounded in the bin's precision),
+    // and it does not retry: many elements for one bin do not starve each
+    // other as compare-and-swap loops would.
+    const F before = unsafeAtomicAdd(static_cast<F*>(bins) + b, (F)1);
+    return checked && before == max_value;
+  }
   U* p = static_cast<U*>(bins) + b;
   U old = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   while (true) {
@@ -182,7 +191,6 @@ __device__ __forceinline__ bool add_to_fp_bin(void* bins, int64_t b, uint32_t c,
   }
   F before;
   __builtin_memcpy(&before, &old, sizeof(F));
-  const F max_value = sizeof(F) == 4 ? (F)3.402823466e+38f : (F)1.7976931348623157e+308;
   return checked && before == max_value;
 }
 

@@ -333,6 +333,15 @@ def test_histogram_floating_point_bins_take_their_ones_in_bin_precision(bin_dtyp
     assert np.isnan(got[7]) and np.isnan(want[7])
     got[7] = want[7] = 0
     assert bits_equal(got, want)
+    # every element for one of many bins: single increments go through the
+    # hardware's floating-point add, which does not retry under contention
+    values = np.full(2000000, 5, dtype=np.int32)
+    got, ov = gpu_histogram(values, np.zeros(nbins, dtype=bin_dtype), capi.LOCATOR_IDENTITY)
+    assert got[5] == 2000000.0 and got.sum() == 2000000.0 and ov == 0
+    start = np.zeros(nbins, dtype=bin_dtype)
+    start[5] = 2.0 ** 24 - 1000
+    got, ov = gpu_histogram(values, start, capi.LOCATOR_IDENTITY)
+    assert got[5] == (2.0 ** 24 if bin_dtype == np.float32 else 2.0 ** 24 + 1999000) and ov == 0
     # modulo locator and float input
     samples = rng.normal(0, 300, 50000).astype(np.float32)
     got, ov = gpu_histogram(samples, np.zeros(64, dtype=bin_dtype), capi.LOCATOR_MODULO)
