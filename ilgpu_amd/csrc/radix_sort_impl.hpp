@@ -431,8 +431,8 @@ __device__ __forceinline__ void load_tile_keys(
 
 // Tile of a group's k-th draw: its chunks are g, g + 8, g + 16, ... of
 // 2^chunk_shift consecutive tiles.
-__device__ __forceinline__ int ticket_tile(uint32_t k, uint32_t g, int chunk_shift) {
-  const uint32_t chunk = (k >> chunk_shift) * kTicketGroups + g;
+__device__ __forceinline__ int ticket_tile(uint32_t k, uint32_t g, uint32_t groups, int chunk_shift) {
+  const uint32_t chunk = (k >> chunk_shift) * groups + g;
   return (int)((chunk << chunk_shift) + (k & ((1u << chunk_shift) - 1u)));
 }
 
@@ -765,7 +765,7 @@ void onesweep_kernel(
     typename ValueOf<VALUE_BYTES>::type* vals_b, int64_t n, int pass,
     KeyXform xf, const uint32_t* __restrict__ excl, uint32_t* status,
     uint32_t* ticket, const SortPlan* __restrict__ plan, int num_tiles,
-    int values_from_index, int chunk_shift, uint32_t spin_limit) {
+    int values_from_index, int groups, int chunk_shift, uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
@@ -814,8 +814,8 @@ void onesweep_kernel(
   // fly while the ranking counters are cleared.
   while (true) {
     if (tid == 0) {
-      const uint32_t g = blockIdx.x % (uint32_t)kTicketGroups;
-      s_tile = ticket_tile(atomicAdd(ticket + g * kTicketStride, 1u), g, chunk_shift);
+      const uint32_t g = blockIdx.x % (uint32_t)groups;
+      s_tile = ticket_tile(atomicAdd(ticket + g * kTicketStride, 1u), g, (uint32_t)groups, chunk_shift);
     }
     __syncthreads();  // also: the previous tile's staged keys have been read
     const int tile = s_tile;
@@ -852,6 +852,691 @@ void onesweep_kernel(
     if (valid != kTile) run(std::false_type{}, std::true_type{});
     else if (hot[0] == kNoHotDigit) run(std::true_type{}, std::false_type{});
     else run(std::true_type{}, std::true_type{});
+  }
+}
+
+// ---- onesweep pass, pipelined form (integer keys only, large inputs) ----------
+// The pass above runs a tile's phases one after the other: while a block waits
+// for its keys nothing else happens on its compute unit, and while it ranks,
+// walks and stages, no load is in flight.  This form overlaps them.
+//
+//   * The write-out of a tile is deferred until the next tile is ranked.  Per
+//     tile: positions and staging of tile T (its keys leave the registers),
+//     load and ranking of the block's next tile T', digit totals of T'
+//     published, T written out from LDS, and so on.  The stores of T drain
+//     while T' is staged and T'' is loaded; T is resolved (the digit counts of
+//     all earlier tiles) while T' is loaded and ranked.
+//   * A 1024-thread block is fifteen waves that sort and one that resolves.
+//     The sorting waves hold the keys (15 x 64 x kItems per tile).  The other
+//     wave holds none and hands the 256 global offsets of a tile over through
+//     LDS.  A wave that sorts could not do this beside its loads: vector memory
+//     results return to a wave, and to a compute unit, in request order, so a
+//     status word asked for behind a tile of keys arrives behind the keys.  For
+//     the same reason a look-back step on a compute unit that streams keys
+//     takes three times what it takes on an idle one, and a walk of the usual
+//     depth (thirty tiles) would outlast the tile.
+//   * So the walking is done elsewhere.  Four blocks of the grid sort nothing:
+//     their compute units issue no key traffic and their memory round trips are
+//     short.  Each takes 64 of the 256 digits and turns the published counts of
+//     the tiles into inclusive prefixes, in tile order, a window of 64 tiles per
+//     round trip.  A sorting block's sixteenth wave only polls the row of its
+//     own tile until the prefixes are there.  Every status row is read by the
+//     scanning blocks and by its owner, not by the thirty tiles behind it.
+//     Nothing waits without bound: a wave that has polled its row often enough
+//     walks back itself (pipelined_walk), and a scanning block that waits for a
+//     tile nobody publishes counts that tile's digits itself.
+//   * A tile's digit counts are published a fixed time after its ticket is
+//     drawn (staging of the previous tile, load, ranking), whatever any other
+//     block does and however long the tile before takes to be resolved: a
+//     ticket commits the block to the tile, and every later tile waits for
+//     those counts.  That is why the sorting waves never meet the sixteenth
+//     wave inside their own steps: among themselves they synchronise through
+//     counters in LDS (arrive: one add by a wave's first lane; wait: poll), and
+//     the block-wide barrier is used once per tile, where the offsets of the
+//     tile before are handed over.
+//   * The ranking counters have LDS of their own (the tile is 1/16 shorter,
+//     which frees it): a wave clears its counters itself as soon as it has read
+//     its run starts, and no barrier separates positions from staging.
+//
+// Floating-point keys and pairs take the pass above.
+template <int KEY_BYTES> struct PipelinedTile {
+  static constexpr int kBlock = 1024;
+  static constexpr int kSorterWaves = kBlock / kWaveSize - 1;
+  static constexpr int kSorters = kSorterWaves * kWaveSize;
+  static constexpr int kItems = items_per_thread(KEY_BYTES, 0);
+  static constexpr int kSubTileKeys = kWaveSize * kItems;
+  static constexpr int kTile = kSorterWaves * kSubTileKeys;
+};
+constexpr int pipelined_tile_keys(int key_bytes) {
+  return (1024 / kWaveSize - 1) * kWaveSize * items_per_thread(key_bytes, 0);
+}
+#ifndef ILGPU_HIP_SORT_WALK_STEP
+#define ILGPU_HIP_SORT_WALK_STEP 4
+#endif
+constexpr int kWalkStep = ILGPU_HIP_SORT_WALK_STEP;   // tiles per look-back step of a resolving wave that walks back itself
+constexpr int kWalkDigits = kRadix / kWaveSize;       // digits per lane of a resolving wave
+
+// Loads the calling wave's keys of one tile into `key` and ranks them on the
+// wave's counters, which are zero on entry: as in sort_tile.
+template <int KEY_BYTES, bool FULL, bool HOT>
+__device__ __forceinline__ void pipelined_rank(
+    typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, 0))],
+    uint32_t (&packed)[(items_per_thread(KEY_BYTES, 0)) / 2],
+    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int64_t tile_base, int valid,
+    int shift, typename KeyOf<KEY_BYTES>::type xor_mask, uint32_t* my_counters, int lane, int first_local,
+    const uint32_t (&hot)[kMaxHot]) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  constexpr int kItems = items_per_thread(KEY_BYTES, 0);
+  load_tile_keys<KEY_BYTES, kItems, FULL>(src_keys, tile_base, valid, first_local, key);
+  auto item_digit = [&](int j) -> uint32_t {
+    const uint32_t d = (uint32_t)((K)(key[j] ^ xor_mask) >> shift) & (kRadix - 1);
+    return (FULL || first_local + j * kWaveSize < valid) ? d : (uint32_t)(kRadix - 1);
+  };
+  uint32_t hot_count[kMaxHot] = {};
+  constexpr int kGroup = ILGPU_HIP_SORT_RANK_GROUP;
+  static_assert(kGroup % 2 == 0, "ranks are packed in pairs");
+#pragma unroll
+  for (int j0 = 0; j0 < kItems; j0 += kGroup) {
+    uint32_t fetched[kGroup];
+    uint32_t offset[kGroup];
+    bool broadcast[kGroup];
+#pragma unroll
+    for (int g = 0; g < kGroup; ++g) {
+      const int j = j0 + g;
+      if (j >= kItems) break;
+      const uint32_t d = item_digit(j);
+      fetched[g] = 0;
+      offset[g] = 0;
+      broadcast[g] = false;
+      bool through_counter = true;
+      if constexpr (HOT) {
+#pragma unroll
+        for (int h = 0; h < kMaxHot; ++h) {
+          if (hot[h] == kNoHotDigit) continue;  // wave-uniform
+          const bool is_hot = d == hot[h];
+          const uint64_t hot_lanes = __ballot(is_hot);
+          if (is_hot) {
+            offset[g] = hot_count[h] + (uint32_t)mbcnt(hot_lanes);
+            through_counter = false;
+          }
+          hot_count[h] += (uint32_t)__popcll(hot_lanes);
+        }
+      } else {
+        const uint32_t row_digit = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+        broadcast[g] = __ballot(d == row_digit) == ~0ull;
+        if (broadcast[g]) {
+          offset[g] = (uint32_t)lane;
+          through_counter = lane == 0;
+        }
+      }
+      if (through_counter)
+        fetched[g] = __hip_atomic_fetch_add(my_counters + d,
+                                            broadcast[g] ? (uint32_t)kWaveSize : 1u,
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+#pragma unroll
+    for (int g = 0; g < kGroup; ++g) {
+      const int j = j0 + g;
+      if (j >= kItems) break;
+      uint32_t rank = fetched[g];
+      if constexpr (!HOT) {
+        if (broadcast[g]) rank = (uint32_t)__builtin_amdgcn_readfirstlane((int)rank);
+      }
+      rank += offset[g];
+      if (j % 2 == 0) packed[j / 2] = rank;
+      else packed[j / 2] |= rank << 16;
+    }
+#pragma unroll
+    for (int g = 0; g < kGroup; g += 2)
+      if (j0 + g < kItems) asm volatile("" : "+v"(packed[(j0 + g) / 2]));
+  }
+  if constexpr (HOT) {
+#pragma unroll
+    for (int h = 0; h < kMaxHot; ++h)  // these counters are untouched so far: still zero
+      if (hot[h] != kNoHotDigit && lane == 0) my_counters[hot[h]] = hot_count[h];
+  }
+}
+
+// A resolving wave that walks back itself: the digit counts of all earlier tiles by
+// look-back, the tile's inclusive counts published, the global offsets of its
+// 256 runs into s_global_off.  Lane l owns digits 4l .. 4l+3, so a tile's
+// status row is one 16-byte load per lane: the time of a look-back step grows
+// with the number of load instructions in it, not with their width.
+typedef uint32_t StatusVec __attribute__((ext_vector_type(4)));
+constexpr int kStatusCoherent = 16;  // cache policy of the buffer operations: sc1, agent scope
+__device__ __forceinline__ StatusVec load_status_row(__amdgpu_buffer_rsrc_t rsrc, int tile,
+                                                      int lane) {
+  return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (tile * kRadix + lane * kWalkDigits) * 4, 0,
+                                               kStatusCoherent);
+}
+
+template <int KEY_BYTES>
+__device__ __forceinline__ void pipelined_walk(
+    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int tile, int shift,
+    typename KeyOf<KEY_BYTES>::type xor_mask, __amdgpu_buffer_rsrc_t status,
+    const uint32_t* __restrict__ excl_row, const uint32_t* s_total, const uint32_t* s_start,
+    uint32_t* s_global_off, int lane, uint32_t spin_limit) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  constexpr int kTile = PipelinedTile<KEY_BYTES>::kTile;
+  static_assert(kWalkDigits == 4, "a lane's digits are one 16-byte vector");
+  auto digit = [&](K k) -> uint32_t {
+    return (uint32_t)((K)(k ^ xor_mask) >> shift) & (kRadix - 1);
+  };
+  const StatusVec my_count = reinterpret_cast<const StatusVec*>(s_total)[lane];
+  const StatusVec my_excl = reinterpret_cast<const StatusVec*>(excl_row)[lane];
+  uint32_t before[kWalkDigits];
+  bool done[kWalkDigits];
+#pragma unroll
+  for (int c = 0; c < kWalkDigits; ++c) {
+    before[c] = 0;
+    done[c] = tile == 0;
+  }
+  for (int t = tile - 1; t >= 0; t -= kWalkStep) {
+    bool all_done = true;
+#pragma unroll
+    for (int c = 0; c < kWalkDigits; ++c) all_done = all_done && done[c];
+    if (__all(all_done)) break;
+    // The loads of a step are unconditional (index clamped) so that they are in
+    // flight together; positions in front of tile 0 read as an empty prefix.
+    StatusVec s[kWalkStep];
+#pragma unroll
+    for (int u = 0; u < kWalkStep; ++u)
+      s[u] = load_status_row(status, t - u < 0 ? 0 : t - u, lane);
+#pragma unroll
+    for (int u = 0; u < kWalkStep; ++u) {
+      if (t - u < 0) s[u] = StatusVec{status_prefix(0u), status_prefix(0u), status_prefix(0u),
+                                      status_prefix(0u)};
+      // Words of tile t - u that this lane still needs and that are empty:
+      // the tile's row is polled until they are there, never without bound.
+      uint32_t polls = 0;
+      while (true) {
+        bool missing = false;
+#pragma unroll
+        for (int c = 0; c < kWalkDigits; ++c) missing = missing || (!done[c] && s[u][c] == 0u);
+        if (!__any(missing)) break;
+        if (polls++ >= spin_limit) {
+          // Nobody has published tile t - u: its owner may not be running.
+          // Count the digits of that (full) tile from the source keys and go
+          // on as if the tile had published its own counts.  Slow, and never
+          // needed while every group of blocks is resident.
+          const K* other = src_keys + (int64_t)(t - u) * kTile;
+          uint32_t cnt[kWalkDigits] = {};
+#pragma unroll 4
+          for (int i = 0; i < kTile; ++i) {
+            K k = other[i];
+            const uint32_t d = digit(k);
+#pragma unroll
+            for (int c = 0; c < kWalkDigits; ++c) cnt[c] += d == (uint32_t)(lane * kWalkDigits + c);
+          }
+#pragma unroll
+          for (int c = 0; c < kWalkDigits; ++c)
+            if (s[u][c] == 0u) s[u][c] = status_aggregate(cnt[c]);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        s[u] = load_status_row(status, t - u, lane);
+      }
+#pragma unroll
+      for (int c = 0; c < kWalkDigits; ++c) {
+        if (!done[c]) {
+          before[c] += status_value(s[u][c]);
+          done[c] = !status_is_aggregate(s[u][c]);
+        }
+      }
+    }
+  }
+  StatusVec prefix, offset;
+  const StatusVec start = reinterpret_cast<const StatusVec*>(s_start)[lane];
+#pragma unroll
+  for (int c = 0; c < kWalkDigits; ++c) {
+    prefix[c] = status_prefix(before[c] + my_count[c]);
+    offset[c] = my_excl[c] + before[c] - start[c];
+  }
+  if (tile > 0)
+    __builtin_amdgcn_raw_buffer_store_b128(prefix, status, (tile * kRadix + lane * kWalkDigits) * 4,
+                                           0, kStatusCoherent);
+  reinterpret_cast<StatusVec*>(s_global_off)[lane] = offset;
+}
+
+#ifndef ILGPU_HIP_SORT_OWN_ROW_SLEEP
+#define ILGPU_HIP_SORT_OWN_ROW_SLEEP 20
+#endif
+// Rows (tiles) a scanning block takes per round trip: four per wave, and as
+// many again requested ahead.  (A wave with more than about 24 dwords per lane
+// in flight stalls: measured.)
+#ifndef ILGPU_HIP_SORT_SCAN_SEG_ROWS
+#define ILGPU_HIP_SORT_SCAN_SEG_ROWS 4
+#endif
+constexpr int kScanSegRows = ILGPU_HIP_SORT_SCAN_SEG_ROWS;
+constexpr int kScanSegs = 16;
+constexpr int kScanWindow = kScanSegs * kScanSegRows;
+constexpr int kScanBlocks = kRadix / kWaveSize;  // one scanning block per 64 digits
+// Polls of its own row before a resolving wave stops waiting for the scanning
+// block and walks back itself.
+constexpr uint32_t kScannerPolls = 64;
+
+// A scanning block's loop: status words of the tiles in order, counts into
+// inclusive prefixes, for the 64 digits of the block (lane = digit).  Wave w
+// takes the rows 4w .. 4w+3 of a window of 64 tiles: one round trip reads the
+// window, the rows that are complete at its front are scanned (four rows per
+// thread in registers, the sixteen waves combined through LDS) and their
+// prefixes written back.  A row's word either adds its count or (tile 0, or a
+// tile whose owner walked back itself) sets the running value.
+// s_lds: 16 + 17 x 64 words.
+template <int KEY_BYTES>
+__device__ __forceinline__ void pipelined_scan(
+    const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int shift,
+    typename KeyOf<KEY_BYTES>::type xor_mask, uint32_t* status, int num_tiles, uint32_t spin_limit,
+    uint32_t* s_lds) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  constexpr int kTile = PipelinedTile<KEY_BYTES>::kTile;
+  uint32_t* s_avail = s_lds;                          // [segments]: leading complete rows of every wave's segment
+  uint32_t* s_part = s_lds + kScanSegs;               // [segments][64]: what a segment's rows do to the running value
+  uint32_t* s_prefix = s_part + kScanSegs * kWaveSize;  // [64]: the running inclusive counts
+  static_assert(kScanSegs * kWaveSize >= kRadix, "the fallback counts 256 digit values in s_part");
+  constexpr uint32_t kAbsolute = 0x80000000u; // a segment that sets the running value
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int wave = tid / kWaveSize;
+  const int quarter = blockIdx.x;  // this block's 64 digits
+  const int seg = wave;            // this wave's rows of the window
+  const int dgt = quarter * kWaveSize + lane;
+  auto combine = [&](uint32_t running, uint32_t part) -> uint32_t {
+    return (part & kAbsolute) ? (part & ~kAbsolute) : running + part;
+  };
+  if (seg == 0) s_prefix[lane] = 0u;
+  __syncthreads();
+  uint32_t polls = 0;
+  int t = 0;
+  uint32_t w[kScanSegRows], w_next[kScanSegRows];
+  bool ahead = false;  // w already holds the window at t
+  auto load_window = [&](int first_tile, uint32_t (&words)[kScanSegRows]) {
+#pragma unroll
+    for (int u = 0; u < kScanSegRows; ++u) {
+      int row = first_tile + seg * kScanSegRows + u;
+      row = row < num_tiles ? row : num_tiles - 1;
+      words[u] = __hip_atomic_load(&status[(int64_t)row * kRadix + dgt], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  while (t < num_tiles) {
+    const int first_row = t + seg * kScanSegRows;
+    // The window was requested by the previous turn if that consumed a whole
+    // window (the scan is behind and the rows are there); the next one is
+    // requested before this one is worked on, so that its round trip runs
+    // beside the scan and ahead of this window's stores.
+    if (!ahead) load_window(t, w);
+    load_window(t + kScanWindow, w_next);
+    int there = 0;  // complete rows at the front of this wave's segment (wave-uniform)
+    bool open = true;
+#pragma unroll
+    for (int u = 0; u < kScanSegRows; ++u) {
+      open = open && first_row + u < num_tiles && __all(w[u] != 0u);
+      there += open ? 1 : 0;
+    }
+    if (lane == 0) s_avail[seg] = (uint32_t)there;
+    __syncthreads();
+    // Complete rows at the front of the window.
+    int avail = 0;
+    {
+      bool full = true;
+#pragma unroll
+      for (int g = 0; g < kScanSegs; ++g) {
+        const int a = (int)s_avail[g];
+        avail += full ? a : 0;
+        full = full && a == kScanSegRows;
+      }
+    }
+    int mine = avail - seg * kScanSegRows;  // rows of this segment that are consumed
+    mine = mine < 0 ? 0 : (mine > kScanSegRows ? kScanSegRows : mine);
+    uint32_t value = 0;
+    bool absolute = false;
+    uint32_t was_aggregate = 0;  // bit u: row u held a count
+#pragma unroll
+    for (int u = 0; u < kScanSegRows; ++u) {
+      if (u < mine) {
+        if (status_is_aggregate(w[u])) {
+          value += w[u] & kStatusCountMask;
+          was_aggregate |= 1u << u;
+        } else {
+          value = w[u] - 1u;
+          absolute = true;
+        }
+      }
+      // From here w[u] is the running value within the segment, and whether it
+      // is already absolute rides in the top bit.
+      w[u] = value | (absolute ? kAbsolute : 0u);
+    }
+    s_part[seg * kWaveSize + lane] = value | (absolute ? kAbsolute : 0u);
+    __syncthreads();
+    uint32_t running = s_prefix[lane];
+    uint32_t base = running;
+#pragma unroll
+    for (int g = 0; g < kScanSegs; ++g) {
+      const uint32_t part = s_part[g * kWaveSize + lane];
+      if (g < seg) base = combine(base, part);
+      running = combine(running, part);
+    }
+#pragma unroll
+    for (int u = 0; u < kScanSegRows; ++u) {
+      if (u < mine && ((was_aggregate >> u) & 1u))
+        __hip_atomic_store(&status[(int64_t)(first_row + u) * kRadix + dgt],
+                           status_prefix(combine(base, w[u])), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();  // the segment results and the running counts have been read
+    if (seg == 0) s_prefix[lane] = running;
+    t += avail;
+    ahead = avail == kScanWindow;
+    if (ahead) {
+#pragma unroll
+      for (int u = 0; u < kScanSegRows; ++u) w[u] = w_next[u];
+    }
+    if (avail != 0) {
+      polls = 0;
+    } else if (polls++ >= spin_limit) {
+      // Nobody has published tile t: its owner may not be running.  Count its
+      // digits from the source keys (a full tile: the last one is left to its
+      // owner) and go on; the owner, if it ever runs, resolves itself.  Slow,
+      // and never needed while every block is resident.
+      if (t == num_tiles - 1) return;
+      if (tid < kRadix) s_part[tid] = 0u;
+      __syncthreads();
+      const K* other = src_keys + (int64_t)t * kTile;
+      for (int i = tid; i < kTile; i += kScanSegs * kWaveSize) {
+        K k = other[i];
+        atomicAdd(&s_part[(uint32_t)((K)(k ^ xor_mask) >> shift) & (kRadix - 1)], 1u);
+      }
+      __syncthreads();
+      if (seg == 0) s_prefix[lane] += s_part[dgt];
+      __syncthreads();
+      ++t;
+      polls = 0;
+    } else {
+      __builtin_amdgcn_s_sleep(2);
+    }
+  }
+}
+
+template <int KEY_BYTES>
+__global__ __launch_bounds__(1024, ILGPU_HIP_SORT_WAVES_PER_EU)
+void onesweep_pipelined_kernel(
+    typename KeyOf<KEY_BYTES>::type* keys_a, typename KeyOf<KEY_BYTES>::type* keys_b, int64_t n,
+    int pass, KeyXform xf, const uint32_t* __restrict__ excl, uint32_t* status, uint32_t* ticket,
+    const SortPlan* __restrict__ plan, int num_tiles, int groups, int chunk_shift,
+    uint32_t spin_limit, int with_scanner) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  using Cfg = PipelinedTile<KEY_BYTES>;
+  constexpr int kTile = Cfg::kTile;
+  constexpr int kItems = Cfg::kItems;
+  constexpr int kSorterWaves = Cfg::kSorterWaves;
+  constexpr int kDigitWaves = kRadix / kWaveSize;
+  constexpr int kDrawThread = kRadix;  // first lane of the first wave without digits
+  static_assert(kItems % 2 == 0 && kTile <= 65536,
+                "ranks and tile positions are packed two to a register");
+
+  __shared__ __attribute__((aligned(16))) K s_keys[kTile];
+  __shared__ __attribute__((aligned(16))) uint32_t s_counter[kSorterWaves * kRadix];
+  // Handed between the sorting waves and the resolving wave, which runs up to a
+  // tile behind: two copies each, by the parity of the block's tile count.
+  __shared__ __attribute__((aligned(16))) uint32_t s_total[2][kRadix];
+  __shared__ __attribute__((aligned(16))) uint32_t s_start[2][kRadix];
+  __shared__ __attribute__((aligned(16))) uint32_t s_global_off[2][kRadix];
+  __shared__ int s_next[2];
+  __shared__ uint32_t s_scan[kDigitWaves];
+  __shared__ uint32_t s_bar[4];
+
+  if (plan->skip[pass]) return;
+  const bool src_alt = plan->src_is_alt[pass] != 0;
+  const K* src_keys = src_alt ? keys_b : keys_a;
+  K* dst_keys = src_alt ? keys_a : keys_b;
+  const int shift = pass * 8;
+  const uint32_t group = blockIdx.x % (uint32_t)groups;
+  uint32_t* my_ticket = ticket + group * kTicketStride;
+  const K xor_mask = (K)xf.xor_mask;
+
+  if (with_scanner && blockIdx.x < kScanBlocks) {
+    // ---- a scanning block: the prefixes of 64 digits ----
+    pipelined_scan<KEY_BYTES>(src_keys, shift, xor_mask, status, num_tiles,
+                                          spin_limit, s_counter);
+    return;
+  }
+  if (threadIdx.x == 0)
+    s_next[0] = ticket_tile(atomicAdd(my_ticket, 1u), group, (uint32_t)groups, chunk_shift);
+  if (threadIdx.x < 4) s_bar[threadIdx.x] = 0u;
+  for (int i = threadIdx.x; i < kSorterWaves * kRadix / 4; i += Cfg::kBlock)
+    reinterpret_cast<uint4*>(s_counter)[i] = make_uint4(0u, 0u, 0u, 0u);
+  __syncthreads();
+  int tile = s_next[0];
+  __syncthreads();  // s_next[0] is written again by the first tile
+  auto is_full = [&](int t) -> bool { return n - (int64_t)t * kTile >= kTile; };
+
+  // Synchronisation.  The block-wide barrier (all sixteen waves) is used once
+  // per tile, where the sixteenth wave hands over: it must never be waited for
+  // inside the sorting waves' steps, or the publication of a tile's counts
+  // would wait for the resolution of the tile before.  Among themselves the
+  // sorting waves meet at counters in LDS: a wave arrives with one add by its
+  // first lane (after its own LDS operations have completed) and, where it
+  // needs the others, polls the counter.  it = tiles this block has finished.
+
+  if (__builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize) == kSorterWaves) {
+    // ---- the resolving wave ----
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    // The status words of this pass as a buffer: 16-byte loads and stores with
+    // the cache policy of an agent-scope atomic.
+    const __amdgpu_buffer_rsrc_t status_rows = __builtin_amdgcn_make_buffer_rsrc(
+        status, 0, num_tiles * kRadix * 4, 0x00027000);
+    uint32_t it = 0;
+    __syncthreads();  // the first tile's totals and run starts are there, or there is no tile
+    while (tile < num_tiles) {
+      const uint32_t par = it & 1u;
+      bool resolved = false;
+      if (!resolved && with_scanner && tile > 0) {
+        // The scanning block turns this tile's counts into prefixes; its row is
+        // polled until it has, but never without bound.
+        const StatusVec my_count = reinterpret_cast<const StatusVec*>(s_total[par])[lane];
+        for (uint32_t polls = 0; polls <= spin_limit && polls < kScannerPolls; ++polls) {
+          __builtin_amdgcn_s_sleep(ILGPU_HIP_SORT_OWN_ROW_SLEEP);
+          const StatusVec row = load_status_row(status_rows, tile, lane);
+          bool all = true;
+#pragma unroll
+          for (int c = 0; c < kWalkDigits; ++c)
+            all = all && row[c] != 0u && !status_is_aggregate(row[c]);
+          if (__all(all)) {
+            const StatusVec my_excl =
+                reinterpret_cast<const StatusVec*>(excl + pass * kRadix)[lane];
+            const StatusVec start = reinterpret_cast<const StatusVec*>(s_start[par])[lane];
+            StatusVec offset;
+#pragma unroll
+            for (int c = 0; c < kWalkDigits; ++c)
+              offset[c] = my_excl[c] + (status_value(row[c]) - my_count[c]) - start[c];
+            reinterpret_cast<StatusVec*>(s_global_off[par])[lane] = offset;
+            resolved = true;
+            break;
+          }
+        }
+      }
+      if (!resolved)
+        pipelined_walk<KEY_BYTES>(src_keys, tile, shift, xor_mask, status_rows,
+                                              excl + pass * kRadix, s_total[par], s_start[par],
+                                              s_global_off[par], lane, spin_limit);
+      __syncthreads();  // this tile is resolved; the next one's totals are there, if there is one
+      tile = s_next[par];
+      ++it;
+    }
+    return;
+  }
+
+  // ---- the sorting waves ----
+  uint32_t hot[kMaxHot];
+#pragma unroll
+  for (int h = 0; h < kMaxHot; ++h) hot[h] = plan->hot[pass][h];
+  auto digit = [&](K k) -> uint32_t {
+    return (uint32_t)((K)(k ^ xor_mask) >> shift) & (kRadix - 1);
+  };
+  auto arrive = [&](int which, int lane) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (lane == 0)
+      __hip_atomic_fetch_add(&s_bar[which], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  auto wait_for = [&](int which, uint32_t target, int lane) {
+    if (lane == 0) {
+      while (__hip_atomic_load(&s_bar[which], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) <
+             target)
+        __builtin_amdgcn_s_sleep(1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  };
+  // Tile-local positions from the run starts, the wave's counters cleared for
+  // the next tile, the keys staged in digit order.
+  auto stage = [&](auto full, K (&key)[kItems], uint32_t (&packed)[kItems / 2], int valid,
+                   uint32_t* my_counters, int lane, int first_local) {
+    constexpr bool kFull = decltype(full)::value;
+    auto item_digit = [&](int j) -> uint32_t {
+      return (kFull || first_local + j * kWaveSize < valid) ? digit(key[j])
+                                                             : (uint32_t)(kRadix - 1);
+    };
+#pragma unroll
+    for (int j = 0; j < kItems; j += 2) {
+      const uint32_t p0 = my_counters[item_digit(j)] + (packed[j / 2] & 0xFFFFu);
+      const uint32_t p1 = my_counters[item_digit(j + 1)] + (packed[j / 2] >> 16);
+      packed[j / 2] = p0 | (p1 << 16);
+      if (j % 8 == 6) __builtin_amdgcn_sched_barrier(0);
+    }
+    reinterpret_cast<uint4*>(my_counters)[lane] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+    for (int j = 0; j < kItems; ++j)
+      s_keys[j % 2 == 0 ? packed[j / 2] & 0xFFFFu : packed[j / 2] >> 16] = key[j];
+  };
+  auto write_out = [&](auto full, int valid, const uint32_t* global_off) {
+    constexpr bool kFull = decltype(full)::value;
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const int i = j * Cfg::kSorters + tid;
+      if (kFull || i < valid) {
+        const K k = s_keys[i];
+        const uint32_t g = global_off[digit(k)] + (uint32_t)i;
+        dst_keys[g] = k;
+      }
+      if (j % ILGPU_HIP_SORT_WRITE_GROUP == ILGPU_HIP_SORT_WRITE_GROUP - 1)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // What follows the ranking of a tile, up to the point where its keys are
+  // staged in LDS: digit totals published, run starts, the hand-over with the
+  // resolving wave, the write-out of the tile before, staging.
+  uint32_t it = 0;       // tiles this block has finished
+  bool pending = false;  // a staged tile waits to be written out
+  auto after_ranking = [&](auto full, K (&key)[kItems], uint32_t (&packed)[kItems / 2],
+                           int valid) {
+    // The thread index is made opaque per tile: see sort_tile.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid / kWaveSize;
+    const int first_local = wave * Cfg::kSubTileKeys + lane;
+    uint32_t* my_counters = s_counter + wave * kRadix;
+    const uint32_t par = it & 1u;
+    arrive(0, lane);  // ranked
+    uint32_t drawn = 0;
+    if (tid < kRadix) {
+      // One thread per digit (waves 0..3): totals over the sub-tiles, published
+      // at once; then the tile-local start of every (sub-tile, digit) run.
+      wait_for(0, (it + 1u) * kSorterWaves, lane);
+      uint32_t count = 0;
+#pragma unroll
+      for (int s = 0; s < kSorterWaves; ++s) count += s_counter[s * kRadix + tid];
+      __hip_atomic_store(&status[(int64_t)tile * kRadix + tid],
+                         tile == 0 ? status_prefix(count) : status_aggregate(count),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_total[par][tid] = count;
+      uint32_t inc = count;
+#pragma unroll
+      for (int s = 1; s < kWaveSize; s <<= 1) {
+        const uint32_t o = shfl_up(inc, s);
+        if (lane >= s) inc += o;
+      }
+      if (lane == kWaveSize - 1) s_scan[wave] = inc;
+      arrive(1, lane);
+      wait_for(1, (it + 1u) * kDigitWaves, lane);
+      uint32_t run = inc - count;
+      for (int w = 0; w < wave; ++w) run += s_scan[w];
+      s_start[par][tid] = run;
+#pragma unroll
+      for (int s = 0; s < kSorterWaves; ++s) {
+        const uint32_t c = s_counter[s * kRadix + tid];
+        s_counter[s * kRadix + tid] = run;
+        run += c;
+      }
+    } else if (tid == kDrawThread) {
+      // The block's next tile is drawn now: its keys are loaded as soon as this
+      // tile is staged, and its counts are published right after their ranking,
+      // whatever the look-back of this tile does.
+      drawn = atomicAdd(my_ticket, 1u);
+    }
+    __syncthreads();  // run starts and totals are there; the tile before is resolved
+    if (pending) write_out(std::true_type{}, kTile, s_global_off[par ^ 1u]);
+    if (tid == kDrawThread) s_next[par] = ticket_tile(drawn, group, (uint32_t)groups, chunk_shift);
+    arrive(2, lane);  // the staged tile has been read
+    wait_for(2, (it + 1u) * kSorterWaves, lane);
+    stage(full, key, packed, valid, my_counters, lane, first_local);
+    pending = true;
+    const int next_tile = s_next[par];
+    ++it;
+    return next_tile;
+  };
+
+  auto full_tiles = [&](auto with_hot) {
+    constexpr bool kHot = decltype(with_hot)::value;
+    if (!(tile < num_tiles && is_full(tile))) return;
+    K key[kItems];
+    uint32_t packed[kItems / 2];
+    {
+      int tid = threadIdx.x;
+      asm volatile("" : "+v"(tid));
+      const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize;
+      pipelined_rank<KEY_BYTES, true, kHot>(
+          key, packed, src_keys, (int64_t)tile * kTile, kTile, shift, xor_mask, s_counter + wave * kRadix,
+          lane, wave * Cfg::kSubTileKeys + lane, hot);
+    }
+    bool ranked = true;
+    while (ranked) {
+      const int next_tile = after_ranking(std::true_type{}, key, packed, kTile);
+      ranked = next_tile < num_tiles && is_full(next_tile);
+      if (ranked) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize;
+        pipelined_rank<KEY_BYTES, true, kHot>(
+            key, packed, src_keys, (int64_t)next_tile * kTile, kTile, shift, xor_mask,
+            s_counter + wave * kRadix, lane, wave * Cfg::kSubTileKeys + lane, hot);
+      }
+      tile = next_tile;
+    }
+  };
+  if (hot[0] == kNoHotDigit) full_tiles(std::false_type{});
+  else full_tiles(std::true_type{});
+  // Here the block's next tile, if any, is the one at the end of the input; it
+  // is the last of its group and so of this block.
+  int last_valid = kTile;
+  if (tile < num_tiles) {
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid / kWaveSize;
+    last_valid = (int)(n - (int64_t)tile * kTile);
+    K key[kItems];
+    uint32_t packed[kItems / 2];
+    pipelined_rank<KEY_BYTES, false, true>(
+        key, packed, src_keys, (int64_t)tile * kTile, last_valid, shift, xor_mask,
+        s_counter + wave * kRadix, lane, wave * Cfg::kSubTileKeys + lane, hot);
+    after_ranking(std::false_type{}, key, packed, last_valid);
+  }
+  __syncthreads();  // the last tile is resolved
+  if (pending) {
+    if (last_valid == kTile) write_out(std::true_type{}, kTile, s_global_off[(it & 1u) ^ 1u]);
+    else write_out(std::false_type{}, last_valid, s_global_off[(it & 1u) ^ 1u]);
   }
 }
 
@@ -1037,9 +1722,10 @@ struct TempLayout {
 
 // Layout for tiles of `block` threads.  Temp views are sized for the small
 // block (more tiles, more status words); the large block's layout fits inside.
-TempLayout make_layout(int64_t n, int key_bytes, int value_bytes, int block = kSortBlock) {
+TempLayout make_layout(int64_t n, int key_bytes, int value_bytes, int block = kSortBlock,
+                       int64_t tile_override = 0) {
   TempLayout L;
-  const int64_t tile = tile_keys(key_bytes, value_bytes, block);
+  const int64_t tile = tile_override > 0 ? tile_override : tile_keys(key_bytes, value_bytes, block);
   L.tiles = div_up(n, tile);
   int64_t off = 0;
   L.alt_keys = off; off += align_up(n * key_bytes, 256);
@@ -1119,6 +1805,9 @@ int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L
   }
   int64_t grid = (int64_t)cus * per_cu;
   if (grid > L.tiles) grid = L.tiles;
+  // Every group of blocks needs a block: a grid below eight blocks (few tiles, or
+  // a device with very few compute units) forms as many groups as it has blocks.
+  const int groups = grid < kTicketGroups ? (int)grid : kTicketGroups;
   // Chunks as long as leave every block of the grid a tile of its own in the
   // first round (short inputs: single tiles, handed out round-robin).
   int chunk_shift = 0;
@@ -1133,7 +1822,43 @@ int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L
                          dim3((unsigned)grid), dim3(BLOCK), 0, stream,
                          keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
                          status, tickets + p * kTicketGroups * kTicketStride, plan, (int)L.tiles,
-                         from_index, chunk_shift, spin_limit);
+                         from_index, groups, chunk_shift, spin_limit);
+    }
+    ILGPU_HIP_CHECK(hipGetLastError());
+  }
+  return ILGPU_HIP_SUCCESS;
+}
+
+// The passes of a keys-only sort in the pipelined form (one block per compute unit).
+template <int KEY_BYTES>
+int32_t launch_passes_pipelined(hipStream_t stream, const SortArgs& a, const TempLayout& L,
+                                char* base, const KeyXform& xf, int cus) {
+  using K = typename KeyOf<KEY_BYTES>::type;
+  K* keys_a = static_cast<K*>(a.keys);
+  K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
+  uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
+  SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
+  uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
+  auto* pass_kernel = onesweep_pipelined_kernel<KEY_BYTES>;
+  int64_t grid = cus;  // 1024 threads and 150 KiB of LDS: one block per compute unit
+  if (grid > L.tiles) grid = L.tiles;
+  const int groups = grid < kTicketGroups ? (int)grid : kTicketGroups;
+  int chunk_shift = 0;
+  while (chunk_shift < kMaxChunkShift && (grid << (chunk_shift + 1)) <= L.tiles) ++chunk_shift;
+  const uint32_t spin_limit = g_sort_spin_limit.load(std::memory_order_relaxed);
+#ifndef ILGPU_HIP_SORT_SCANNER
+#define ILGPU_HIP_SORT_SCANNER 1
+#endif
+  // One block scans instead of sorting when the grid can spare it.
+  const int with_scanner = ILGPU_HIP_SORT_SCANNER && grid >= 64 ? 1 : 0;
+  for (int p = 0; p < KEY_BYTES; ++p) {
+    uint32_t* status =
+        reinterpret_cast<uint32_t*>(base + L.status + (int64_t)p * L.status_stride);
+    {
+      ProfileScope scope(stream, "sort_onesweep");
+      hipLaunchKernelGGL(pass_kernel, dim3((unsigned)grid), dim3(1024), 0, stream, keys_a, keys_b,
+                         a.n, p, xf, excl, status, tickets + p * kTicketGroups * kTicketStride,
+                         plan, (int)L.tiles, groups, chunk_shift, spin_limit, with_scanner);
     }
     ILGPU_HIP_CHECK(hipGetLastError());
   }
@@ -1167,8 +1892,16 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   const bool use_large =
       div_up(a.n, (int64_t)tile_keys(KEY_BYTES, VALUE_BYTES, kSortBlockLarge)) >=
       min_tiles_per_cu * cus;
+  const KeyXform xf = make_xform(a.key_type, a.flags);
+#ifndef ILGPU_HIP_SORT_PIPELINED
+#define ILGPU_HIP_SORT_PIPELINED 1
+#endif
+  // Large keys-only sorts of integer keys take the pipelined form of the pass.
+  const bool use_pipelined = ILGPU_HIP_SORT_PIPELINED && VALUE_BYTES == 0 && use_large &&
+                             (xf.reference_term | xf.total_term) == 0;
   const TempLayout L =
-      make_layout(a.n, KEY_BYTES, VALUE_BYTES, use_large ? kSortBlockLarge : kSortBlock);
+      make_layout(a.n, KEY_BYTES, VALUE_BYTES, use_large ? kSortBlockLarge : kSortBlock,
+                  use_pipelined ? pipelined_tile_keys(KEY_BYTES) : 0);
   char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)a.temp, 256));
   K* keys_a = static_cast<K*>(a.keys);
   K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
@@ -1177,7 +1910,6 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
   SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
   uint32_t* hist = reinterpret_cast<uint32_t*>(base + L.hist);
-  const KeyXform xf = make_xform(a.key_type, a.flags);
   const int passes = KEY_BYTES;
   const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
 
@@ -1211,7 +1943,10 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   }
   ILGPU_HIP_CHECK(hipGetLastError());
 
-  if (use_large)
+  if (use_pipelined) {
+    if constexpr (VALUE_BYTES == 0)
+      rc = launch_passes_pipelined<KEY_BYTES>(stream, a, L, base, xf, cus);
+  } else if (use_large)
     rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlockLarge>(stream, a, L, base, xf, cus);
   else
     rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlock>(stream, a, L, base, xf, cus);

@@ -8,3 +8,4 @@ int32_t launch_sort_key_bytes_4(hipStream_t stream, const SortArgs& a) {
 }
 
 }  // namespace ilgpu_hip
+

@@ -832,6 +832,45 @@ def test_sort_with_large_blocks_matches_oracle(large_sort_blocks, dtype, descend
                           O.radix_sort(keys, descending=descending)), n
 
 
+@pytest.mark.parametrize("dtype", [np.uint32, np.int32, np.uint64, np.int64, np.uint16, np.uint8])
+def test_sort_with_scanning_blocks_matches_numpy(large_sort_blocks, dtype):
+    # Integer keys in 1024-thread blocks take the pipelined form of the pass.
+    # From 64 tiles on, four blocks of the grid scan the tiles' digit counts
+    # instead of sorting; below that every block resolves its tiles itself.
+    # Sizes: some 100 tiles and a ragged last one; keys uniform, few-valued
+    # (dominant digits), in runs (whole rows of one digit) and constant.
+    items = 18 if np.dtype(dtype).itemsize == 8 else 36
+    tile = 15 * 64 * items
+    for n in [63 * tile, 64 * tile + 1, 101 * tile + 12345]:
+        note("pipelined sort", np.dtype(dtype).name, n)
+        keys = random_ints(dtype, n, seed=n & 0xFFFF)
+        assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable")), n
+    n = 90 * tile + 777
+    info = np.iinfo(dtype)
+    few = random_ints(np.int64, n, seed=3, lo=0, hi=2).astype(dtype) * (info.max // 3)
+    assert np.array_equal(gpu_sort(few, descending=True), np.sort(few, kind="stable")[::-1])
+    runs = ((np.arange(n, dtype=np.uint64) // 1000) * 2654435761 % (int(info.max) // 2 + 1)).astype(dtype)
+    assert np.array_equal(gpu_sort(runs), np.sort(runs, kind="stable"))
+    const = np.full(n, info.max // 5, dtype=dtype)
+    assert np.array_equal(gpu_sort(const), const)
+
+
+def test_sort_with_scanning_blocks_never_waits_without_bound(large_sort_blocks):
+    # With the bound on polls at zero the scanning blocks count every tile they
+    # find unpublished themselves, and the sorting blocks stop waiting for them
+    # at once and walk back themselves, counting in turn what they find missing.
+    capi.sort_set_parameter(capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT, 0)
+    try:
+        for dtype, tiles in [(np.uint32, 70), (np.uint64, 66), (np.uint8, 65)]:
+            items = 18 if np.dtype(dtype).itemsize == 8 else 36
+            n = tiles * 15 * 64 * items + 31
+            note("pipelined sort, zero spin limit", np.dtype(dtype).name, n)
+            keys = random_ints(dtype, n, seed=tiles)
+            assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable")), n
+    finally:
+        capi.sort_set_parameter(capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT, -1)
+
+
 @pytest.mark.parametrize("key_dtype,value_dtype", [
     (np.uint32, np.uint32), (np.uint64, np.uint32), (np.uint32, np.uint64), (np.int64, np.float64),
     (np.uint8, np.uint8), (np.int16, np.uint16), (np.float32, np.int32), (np.float16, np.uint64)])
