@@ -37,6 +37,7 @@ namespace ILGPU.Algorithms.Hip
             int keyType, int valueBytes, int flags, int valueSource, void* temp, long tempBytes);
         [DllImport(LibName)] internal static extern int ilgpu_hip_selftest_lds_atomic_order(
             IntPtr stream, int rows, long* mismatches);
+        [DllImport(LibName)] internal static extern int ilgpu_hip_sort_check_device(IntPtr stream);
         [DllImport(LibName)] internal static extern int ilgpu_hip_sort_set_parameter(
             int parameter, int value);
 

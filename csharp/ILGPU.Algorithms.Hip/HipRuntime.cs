@@ -169,6 +169,13 @@ namespace ILGPU.Algorithms.Hip
             Device = device;
             HipRuntimeNativeMethods.Check(HipRuntimeNativeMethods.hipSetDevice(device));
             DefaultStream = new HipStream(IntPtr.Zero, owned: false);
+            // The sort ranks keys with returning LDS atomics and needs their lanes
+            // served in lane order; the library asks every device once.  Asked
+            // here, the answer is there before any sort (also one on a stream
+            // that is being captured, which could not wait for it), and a device
+            // that fails is refused at construction (NotSupportedException).
+            HipAlgorithmsException.ThrowIfFailed(
+                HipAlgorithmsNativeMethods.ilgpu_hip_sort_check_device(IntPtr.Zero));
         }
 
         public int Device { get; }

@@ -45,7 +45,8 @@ EXPORTS = [
     "ilgpu_hip_profile_query", "ilgpu_hip_radix_sort_temp_bytes",
     "ilgpu_hip_radix_sort_temp_bytes_strided",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
-    "ilgpu_hip_selftest_lds_atomic_order", "ilgpu_hip_sort_set_parameter",
+    "ilgpu_hip_selftest_lds_atomic_order", "ilgpu_hip_sort_check_device",
+    "ilgpu_hip_sort_set_parameter",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan", "ilgpu_hip_scan_static",
     "ilgpu_hip_reduce_temp_bytes", "ilgpu_hip_reduce", "ilgpu_hip_histogram",
     "ilgpu_hip_unique_temp_bytes", "ilgpu_hip_unique", "ilgpu_hip_initialize",
@@ -133,6 +134,8 @@ def lib() -> ctypes.CDLL:
             vp, vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, i64]
         L.ilgpu_hip_selftest_lds_atomic_order.argtypes = [vp, i32, vp]
         L.ilgpu_hip_selftest_lds_atomic_order.restype = i32
+        L.ilgpu_hip_sort_check_device.argtypes = [vp]
+        L.ilgpu_hip_sort_check_device.restype = i32
         L.ilgpu_hip_sort_set_parameter.argtypes = [i32, i32]
         L.ilgpu_hip_sort_set_parameter.restype = i32
         L.ilgpu_hip_scan_temp_bytes.argtypes = [i64, i32, p64]
@@ -317,16 +320,26 @@ def selftest_lds_atomic_order(rows: int = 256, *, stream=None) -> int:
     return int(out.numpy()[0])
 
 
+def sort_check_device(*, stream=None) -> None:
+    """Asks the current device once whether its LDS serves the lanes of an atomic
+    in lane order (what every sort does first); raises NotSupportedError for a
+    device that does not."""
+    check(lib().ilgpu_hip_sort_check_device(_stream_ptr(stream)))
+
+
 SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0
 SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1
 SORT_PARAM_ONE_TILE_KERNEL = 2
+SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER = 3
 
 
 def sort_set_parameter(parameter: int, value: int) -> None:
     """Process-wide sort parameter; a negative value restores the default.
     LOOKBACK_SPIN_LIMIT: polls of an empty status word before a pass counts a
     missing tile itself (0 = at once: exercises the slow path).
-    LARGE_BLOCK_MIN_TILES_PER_CU: 0 = always 1024-thread blocks, 2^31-1 = never."""
+    LARGE_BLOCK_MIN_TILES_PER_CU: 0 = always 1024-thread blocks, 2^31-1 = never.
+    ASSUME_LDS_ATOMIC_ORDER: 0 / 1 = every device counts as having failed / passed
+    the check that precedes every sort; negative = ask the devices (anew)."""
     check(lib().ilgpu_hip_sort_set_parameter(parameter, value))
 
 

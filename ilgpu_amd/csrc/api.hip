@@ -283,10 +283,15 @@ int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
                                           mismatches);
 }
 
+int32_t ilgpu_hip_sort_check_device(ilgpu_hip_stream_t stream) {
+  return check_sort_device(static_cast<hipStream_t>(stream));
+}
+
 int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value) {
   if (parameter != ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT &&
       parameter != ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU &&
-      parameter != ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL)
+      parameter != ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL &&
+      parameter != ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER)
     return ILGPU_HIP_ERROR_OUT_OF_RANGE;
   set_sort_parameter(parameter, value);
   return ILGPU_HIP_SUCCESS;

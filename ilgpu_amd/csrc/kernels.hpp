@@ -56,6 +56,11 @@ void set_sort_parameter(int32_t parameter, int32_t value);
 // returning LDS atomic that share an address are served in lane order.
 // mismatches[0] (device) receives the number of lanes found out of order.
 int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* mismatches);
+// The same check once per device, with the answer kept: SUCCESS, or
+// NOT_SUPPORTED for a device that serves the lanes in another order (or while
+// `stream` is being captured and the device has not been asked yet).  Every
+// sort calls it first.
+int32_t check_sort_device(hipStream_t stream);
 
 // scan.hip: Unique (consecutive duplicates removed in place, new length to
 // out_length[0] on the device).

@@ -9,6 +9,9 @@ namespace ilgpu_hip {
 std::atomic<uint32_t> g_sort_spin_limit{kDefaultSpinLimit};
 std::atomic<int32_t> g_sort_large_min_tiles_per_cu{-1};
 std::atomic<int32_t> g_sort_small_kernel{1};
+// Test hook: -1 = ask the device (the default), 0 / 1 = every device is taken
+// to have failed / passed the check of its LDS atomics.
+std::atomic<int32_t> g_sort_assume_lds_order{-1};
 
 // radix_sort_k<bytes>.hip
 int32_t launch_sort_key_bytes_1(hipStream_t stream, const SortArgs& a);
@@ -55,6 +58,12 @@ __global__ __launch_bounds__(kSortBlock) void lds_atomic_order_kernel(
   if (wrong != 0) atomicAdd(mismatches, wrong);
 }
 
+
+// What the check found, per device: 0 = not asked yet, 1 = lanes served in
+// order, 2 = not.  The counter the check kernels add to is a device array of
+// the library, so the check allocates nothing.
+std::atomic<int> g_lds_order_state[kMaxCachedDevices];
+__device__ __align__(8) unsigned long long g_lds_order_mismatches[2];
 
 // ---- strided views ------------------------------------------------------------
 // Stride1D.General with an element stride above one: the view is gathered
@@ -120,7 +129,11 @@ int32_t launch_dense(hipStream_t stream, const SortArgs& a) {
 }  // namespace
 
 void set_sort_parameter(int32_t parameter, int32_t value) {
-  if (parameter == ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT)
+  if (parameter == ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER) {
+    g_sort_assume_lds_order.store(value < 0 ? -1 : (value == 0 ? 0 : 1), std::memory_order_relaxed);
+    if (value < 0)  // and ask the devices again
+      for (auto& state : g_lds_order_state) state.store(0, std::memory_order_relaxed);
+  } else if (parameter == ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT)
     g_sort_spin_limit.store(value < 0 ? kDefaultSpinLimit : (uint32_t)value, std::memory_order_relaxed);
   else if (parameter == ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU)
     g_sort_large_min_tiles_per_cu.store(value < 0 ? -1 : value, std::memory_order_relaxed);
@@ -142,6 +155,40 @@ int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* 
   return ILGPU_HIP_SUCCESS;
 }
 
+// Every sort goes through here first.  The ranking of a pass is stable only if
+// the lanes of one returning LDS atomic that meet in one address are served in
+// lane order, which the hardware does and no document promises: the first sort
+// on a device plays the check kernels once (some tens of microseconds and one
+// wait for the stream) and the answer is kept per device; a device that fails
+// is refused rather than sorted wrongly.
+int32_t check_sort_device(hipStream_t stream) {
+  const int32_t assumed = g_sort_assume_lds_order.load(std::memory_order_relaxed);
+  if (assumed >= 0) return assumed ? ILGPU_HIP_SUCCESS : ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int device = current_device();
+  std::atomic<int>* state =
+      device >= 0 && device < kMaxCachedDevices ? &g_lds_order_state[device] : nullptr;
+  const int known = state ? state->load(std::memory_order_acquire) : 0;
+  if (known == 1) return ILGPU_HIP_SUCCESS;
+  if (known == 2) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  // The answer has to come back to the host, which a stream that is being
+  // captured cannot give: such callers check the device before they capture.
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+      capturing != hipStreamCaptureStatusNone)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  void* counter = nullptr;
+  ILGPU_HIP_CHECK(hipGetSymbolAddress(&counter, HIP_SYMBOL(g_lds_order_mismatches)));
+  const int32_t rc =
+      launch_lds_atomic_order_selftest(stream, 64, static_cast<int64_t*>(counter));
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  unsigned long long mismatches = ~0ull;
+  ILGPU_HIP_CHECK(hipMemcpyAsync(&mismatches, counter, sizeof(mismatches), hipMemcpyDeviceToHost,
+                                 stream));
+  ILGPU_HIP_CHECK(hipStreamSynchronize(stream));
+  if (state) state->store(mismatches == 0 ? 1 : 2, std::memory_order_release);
+  return mismatches == 0 ? ILGPU_HIP_SUCCESS : ILGPU_HIP_ERROR_NOT_SUPPORTED;
+}
+
 int64_t radix_sort_max_length() { return kMaxSortLength; }
 
 int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
@@ -156,6 +203,8 @@ int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,
 }
 
 int32_t launch_radix_sort(hipStream_t stream, const SortArgs& a) {
+  const int32_t checked = check_sort_device(stream);
+  if (checked != ILGPU_HIP_SUCCESS) return checked;
   const bool has_values = a.values != nullptr && a.value_bytes > 0;
   const bool keys_strided = a.key_stride != 1;
   const bool values_strided = has_values && a.value_stride != 1;

@@ -204,6 +204,10 @@ class Accelerator {
  public:
   explicit Accelerator(int device = 0) : device_(device), default_(nullptr, false) {
     CheckHip(hipSetDevice(device));
+    // The sort needs the lanes of an LDS atomic served in lane order; the
+    // library asks every device once.  Asked here, the answer is there before
+    // any sort, and a device that fails is refused (NotSupportedException).
+    HipAlgorithmsException::ThrowIfFailed(ilgpu_hip_sort_check_device(nullptr));
   }
   AcceleratorStream& DefaultStream() { return default_; }
   std::unique_ptr<AcceleratorStream> CreateStream() {

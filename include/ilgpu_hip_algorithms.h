@@ -189,10 +189,26 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void *keys,
 int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
                                             int32_t rows, int64_t *mismatches);
 
-/* Two process-wide parameters of the sort, for tests and tuning; they apply to
- * sorts launched afterwards, a negative value restores the default, and neither
- * has a counterpart in the reference (its passes are separate kernel launches,
- * RadixSortExtensions.cs:1276-1334).
+/* The same check, once per device and with the answer kept by the library:
+ * ILGPU_HIP_SUCCESS for a device whose LDS serves the lanes in order,
+ * ILGPU_HIP_ERROR_NOT_SUPPORTED for one that does not.  Every sort entry point
+ * calls it first, so no sort runs on a device that has not passed: the first
+ * sort on a device plays the check kernels (64 rows) on a counter inside the
+ * library (nothing is allocated) and waits for `stream` once; later calls cost
+ * one atomic load.  A stream that is being captured cannot be waited for: on a
+ * device that has not been asked yet, a sort on such a stream (and this call)
+ * returns ILGPU_HIP_ERROR_NOT_SUPPORTED, so callers that capture call this
+ * first, outside the capture; accelerator objects of the host layers call it
+ * in their constructors.  No counterpart in the reference. */
+int32_t ilgpu_hip_sort_check_device(ilgpu_hip_stream_t stream);
+
+/* TEST HOOK, not part of the product surface: process-wide parameters of the
+ * sort for the library's own tests and tuning runs.  They are global mutable
+ * state (a thread that changes one changes every sort of the process that is
+ * launched afterwards), so applications leave them alone and bindings keep
+ * them out of their public surface.  A negative value restores the default;
+ * none has a counterpart in the reference (its passes are separate kernel
+ * launches, RadixSortExtensions.cs:1276-1334).
  *   LOOKBACK_SPIN_LIMIT  how often the look-back of a pass polls the status
  *     word of an earlier tile that has published nothing before it stops
  *     waiting and counts that tile's digit itself from the source keys (tiles
@@ -209,11 +225,16 @@ int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
  *   ONE_TILE_KERNEL  inputs of at most one 512-thread tile (18432 keys of up
  *     to 4 bytes, fewer for wider keys and for pairs) are sorted by one block
  *     in one launch, without temp memory.  Default 1; 0 sends them through
- *     the passes like longer inputs. */
+ *     the passes like longer inputs.
+ *   ASSUME_LDS_ATOMIC_ORDER  what ilgpu_hip_sort_check_device answers: 0 = every
+ *     device is taken to have failed the check (sorts return
+ *     ILGPU_HIP_ERROR_NOT_SUPPORTED before anything is launched), 1 = taken to
+ *     have passed, negative (the default) = the devices are asked, anew. */
 enum {
   ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0,
   ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1,
-  ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL = 2
+  ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL = 2,
+  ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER = 3
 };
 int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value);
 

@@ -27,3 +27,18 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _sort_parameters_at_their_defaults():
+    """The sort's test hooks are process-wide: whatever a test sets (or leaves
+    set when it fails half way) is put back before the next test runs."""
+    yield
+    try:
+        from ilgpu_amd import capi
+    except Exception:
+        return
+    for parameter in (capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT,
+                      capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU,
+                      capi.SORT_PARAM_ONE_TILE_KERNEL):
+        capi.lib().ilgpu_hip_sort_set_parameter(parameter, -1)

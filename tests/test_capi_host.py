@@ -196,3 +196,39 @@ def test_transform_argument_validation():
     assert rcall(n_out=8) == capi.ERROR_OUT_OF_RANGE
     assert rcall(n=(1 << 31), n_order=(1 << 31), n_out=(1 << 31)) == capi.ERROR_NOT_SUPPORTED  # :166-170
     assert rcall(st=capi.F16, tt=capi.U8) == capi.ERROR_NOT_SUPPORTED
+
+
+def test_no_sort_runs_on_a_device_that_failed_the_lds_atomic_check():
+    # Every sort asks first whether the device serves the lanes of an LDS atomic
+    # in lane order (the ranking of a pass rests on it) and keeps the answer per
+    # device.  The test hook stands in for a device that fails: both sort entry
+    # points and the query itself answer NOT_SUPPORTED before anything is
+    # launched, so this needs no GPU and the pointers are never touched.
+    L = capi.lib()
+    n = 1000
+    keys, values, temp = (ctypes.c_void_p(0x10000), ctypes.c_void_p(0x20000),
+                          ctypes.c_void_p(0x40000))
+    temp_bytes = capi.radix_sort_temp_bytes(n, np.uint32, 4)
+
+    def sort_keys():
+        return L.ilgpu_hip_radix_sort_keys(None, keys, n, 1, capi.U32, 0, temp, temp_bytes)
+
+    def sort_pairs():
+        return L.ilgpu_hip_radix_sort_pairs(None, keys, 1, values, 1, n, capi.U32, 4, 0,
+                                            capi.VALUES_FROM_VIEW, temp, temp_bytes)
+
+    capi.sort_set_parameter(capi.SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER, 0)
+    try:
+        assert L.ilgpu_hip_sort_check_device(None) == capi.ERROR_NOT_SUPPORTED
+        assert sort_keys() == capi.ERROR_NOT_SUPPORTED
+        assert sort_pairs() == capi.ERROR_NOT_SUPPORTED
+        with pytest.raises(capi.NotSupportedError):
+            capi.check(L.ilgpu_hip_sort_check_device(None))
+        # argument checks still come first
+        assert L.ilgpu_hip_radix_sort_keys(None, None, n, 1, capi.U32, 0, temp,
+                                           temp_bytes) == capi.ERROR_NULL_VIEW
+        # a device that is taken to have passed is not asked either
+        capi.sort_set_parameter(capi.SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER, 1)
+        assert L.ilgpu_hip_sort_check_device(None) == capi.SUCCESS
+    finally:
+        capi.sort_set_parameter(capi.SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER, -1)

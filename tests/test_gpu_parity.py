@@ -703,6 +703,25 @@ def test_lds_atomics_serve_the_lanes_of_an_instruction_in_lane_order():
         capi.selftest_lds_atomic_order(0)
 
 
+def test_sorts_ask_the_device_once_and_refuse_one_that_fails():
+    # The library runs the check of the LDS atomics itself before the first sort
+    # on a device and keeps the answer.
+    capi.sort_set_parameter(capi.SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER, -1)   # forget, ask again
+    keys = random_ints(np.uint32, 50000, seed=1)
+    assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))   # asks the device
+    capi.sort_check_device()                                               # cached: passes
+    capi.sort_set_parameter(capi.SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER, 0)    # stand-in for a device that fails
+    try:
+        with pytest.raises(capi.NotSupportedError):
+            gpu_sort(keys)
+        values = np.arange(keys.size, dtype=np.uint32)
+        with pytest.raises(capi.NotSupportedError):
+            gpu_sort_pairs(keys, values)
+    finally:
+        capi.sort_set_parameter(capi.SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER, -1)
+    assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+
+
 def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
     # A pass hands its tiles to eight fixed groups of blocks, so a tile's
     # look-back can meet a predecessor nobody has started; past a bound of polls
