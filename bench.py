@@ -92,15 +92,21 @@ CSRC = os.path.join(ROOT, "ilgpu_amd", "csrc")
 
 
 def source_digest(file_name):
-    """Digest of a kernel source's code: // comments, indentation and blank
-    lines do not count, so that only a change of code makes the counters stale."""
+    """Digest of what a kernel is built from: the code of its source file and of
+    the headers every kernel file includes, and the compiler flags.  // comments,
+    indentation and blank lines do not count, so that only a change of code (or
+    of the build) makes the counters stale."""
     import hashlib
-    lines = []
-    with open(os.path.join(CSRC, file_name), encoding="utf-8") as f:
-        for line in f:
-            code = line.split("//", 1)[0].strip()
-            if code:
-                lines.append(code)
+    from ilgpu_amd import build
+    lines = list(build.FLAGS)
+    for name in (file_name, "common.hpp", "kernels.hpp"):
+        if name != file_name and not os.path.exists(os.path.join(CSRC, name)):
+            continue
+        with open(os.path.join(CSRC, name), encoding="utf-8") as f:
+            for line in f:
+                code = line.split("//", 1)[0].strip()
+                if code:
+                    lines.append(code)
     return hashlib.sha256("\n".join(lines).encode()).hexdigest()[:16]
 
 
@@ -181,7 +187,7 @@ def main():
                  ("zero_words", "sort_histogram", "sort_plan", "sort_onesweep",
                   "sort_finish")}
     capi.profile_enable(False)
-    passes = pass_launches // K if K else 0
+    passes, _ = capi.radix_sort_passes(temp, n, np.uint32)   # executed, from the sort's plan
     pass_bytes = 2.0 * n * 4            # read + write of the keys, one pass
     pass_gbs = pass_bytes / (pass_ms * 1e-3) / 1e9 if pass_ms else 0.0
     sort_bytes = n * 4.0 * (2 * passes + 1)
@@ -404,6 +410,42 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
         del sk, rk, rv, gk, gv
     del k64, wk, wv, dk, dv, temp, flip
 
+    # Sizes between one tile and the headline: 2^20 (the configuration the
+    # reference's CPUAccelerator can run: compared bit for bit with the oracle
+    # at full size), 2^22 and 2^24.  At these sizes the launches count: the
+    # entry says how many kernels one sort launches.
+    if cpu_on:
+        for log2m in (20, 22, 24):
+            m = 1 << log2m
+            part = datagen.uniform_u32_torch(m)
+            wk = torch.empty_like(part)
+            kv = wrap(wk, np.uint32)
+            tp = capi.temp_buffer(capi.radix_sort_temp_bytes(m, np.uint32))
+            ms, _ = timer.run(lambda: wk.copy_(part), lambda: capi.radix_sort_keys(kv, tp), K, W)
+            capi.profile_enable(True)
+            timer.run(lambda: wk.copy_(part), lambda: capi.radix_sort_keys(kv, tp), 1, 0)
+            launches = sum(kernel_stats(capi, k)[0] for k in
+                           ("zero_words", "sort_histogram", "sort_plan", "sort_onesweep",
+                            "sort_finish", "sort_small"))
+            capi.profile_enable(False)
+            t = float(np.median(ms))
+            host = part.cpu().numpy().view(np.uint32)
+            t0 = time.perf_counter(); ref = O.radix_sort(host); dt = time.perf_counter() - t0
+            ok = bool(np.array_equal(wk.cpu().numpy().view(np.uint32), ref))
+            passes, _ = capi.radix_sort_passes(tp, m, np.uint32)
+            algo = m * 4.0 * (2 * passes + 1)
+            out[f"radix_sort_u32_2^{log2m}"] = {
+                "ms_per_step": round(t, 4), "gkeys_per_s": round(m / (t * 1e-3) / 1e9, 2),
+                "passes_executed": passes, "kernel_launches": launches,
+                "algorithmic_gbs": round(algo / (t * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(algo / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "verified": ok,
+                "cpu_baseline": {"value": round(m / dt / 1e9, 5), "unit": "Gkeys/s", "cores": 1,
+                                 "kind": "port", "sample": f"all 2^{log2m} keys, {dt:.1f} s"}}
+            log(f"[bench] radix_sort_u32_2^{log2m}: {t:.4f} ms/step, "
+                f"{m / (t * 1e-3) / 1e9:.1f} Gkeys/s, {launches} launches, verified={ok}")
+            del part, wk, kv, tp, host, ref
+
     # Skewed sorts: Zipf(1.1) over 2^16 values, and all keys equal
     for name, src in (("radix_sort_u32_zipf_2^28", datagen.zipf_u32_torch(n28)),
                       ("radix_sort_u32_all_equal_2^28",
@@ -419,7 +461,7 @@ def run_extras(args, torch, capi, datagen, timer, wrap):
         o64 = work.to(torch.int64) & 0xFFFFFFFF
         ok = bool((o64[1:] >= o64[:-1]).all().item()) and \
             int(o64.sum().item()) == int((src.to(torch.int64) & 0xFFFFFFFF).sum().item())
-        passes = 2 if "zipf" in name else 0
+        passes, _ = capi.radix_sort_passes(temp, n28, np.uint32)   # read from the sort's plan
         algo = n28 * 4.0 * (2 * passes + 1)
         out[name] = {"ms_per_step": round(t, 4),
                      "gkeys_per_s": round(n28 / (t * 1e-3) / 1e9, 2),

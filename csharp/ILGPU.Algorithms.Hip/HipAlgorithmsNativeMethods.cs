@@ -35,6 +35,9 @@ namespace ILGPU.Algorithms.Hip
         [DllImport(LibName)] internal static extern int ilgpu_hip_radix_sort_pairs(
             IntPtr stream, void* keys, long keyStride, void* values, long valueStride, long n,
             int keyType, int valueBytes, int flags, int valueSource, void* temp, long tempBytes);
+        [DllImport(LibName)] internal static extern int ilgpu_hip_radix_sort_passes(
+            IntPtr stream, void* temp, long tempBytes, long n, int keyType, int valueBytes,
+            out int executed, out int skipped);
         [DllImport(LibName)] internal static extern int ilgpu_hip_selftest_lds_atomic_order(
             IntPtr stream, int rows, long* mismatches);
         [DllImport(LibName)] internal static extern int ilgpu_hip_sort_check_device(IntPtr stream);

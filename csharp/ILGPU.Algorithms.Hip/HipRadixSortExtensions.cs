@@ -67,6 +67,79 @@ namespace ILGPU.Algorithms.Hip
             return checked((int)HipTypeMap.BytesToInts(bytes));
         }
 
+        /// <summary>The temp size, in 32-bit integers, of a sort of views with element
+        /// strides above one (the strided views are gathered into a dense copy at
+        /// the end of temp, sorted there and scattered back); valueBytes is 0 for
+        /// keys only.  The reference's sizing helpers have no stride argument.</summary>
+        public static LongIndex1D ComputeRadixSortTempStorageSize<T, TRadixSortOperation>(
+            this HipAccelerator accelerator,
+            LongIndex1D dataLength,
+            int valueBytes,
+            long keyStride,
+            long valueStride)
+            where T : unmanaged
+            where TRadixSortOperation : struct, IRadixSortOperation<T>
+        {
+            var (keyType, _) = HipTypeMap.SortOperation<T, TRadixSortOperation>();
+            HipAlgorithmsException.ThrowIfFailed(
+                ilgpu_hip_radix_sort_temp_bytes_strided(
+                    dataLength, keyType, valueBytes, keyStride, valueStride, out long bytes),
+                nameof(dataLength));
+            return HipTypeMap.BytesToInts(bytes);
+        }
+
+        /// <summary>How many 8-bit passes the last sort that used temp ran and how
+        /// many it found unnecessary (a pass whose digit is the same for every key
+        /// is skipped); same length, key type and value size (0 for keys only) as
+        /// that sort.  Waits for the stream.  The reference runs every pass whatever
+        /// the keys and has nothing to report.</summary>
+        public static (int Executed, int Skipped) GetRadixSortPasses<T, TRadixSortOperation>(
+            this HipAccelerator accelerator,
+            AcceleratorStream stream,
+            ArrayView<int> temp,
+            LongIndex1D dataLength,
+            int valueBytes = 0)
+            where T : unmanaged
+            where TRadixSortOperation : struct, IRadixSortOperation<T>
+        {
+            var (keyType, _) = HipTypeMap.SortOperation<T, TRadixSortOperation>();
+            CheckTemp(temp);
+            HipAlgorithmsException.ThrowIfFailed(
+                ilgpu_hip_radix_sort_passes(
+                    HipStream.PtrOf(stream),
+                    temp.LoadEffectiveAddressAsPtr().ToPointer(),
+                    temp.Length * sizeof(int),
+                    dataLength,
+                    keyType,
+                    valueBytes,
+                    out int executed,
+                    out int skipped),
+                nameof(temp));
+            return (executed, skipped);
+        }
+
+        /// <summary>The library's own check of the one hardware property the ranking
+        /// of a pass rests on (lanes of one LDS atomic served in lane order), played
+        /// over `rows` rows per wave: the number of lanes found out of order, 0 on
+        /// gfx950.  Every sort runs a short form of it once per device by itself
+        /// (HipAccelerator's constructor asks for it); this is the long form for
+        /// diagnostics.</summary>
+        public static long CountLdsAtomicOrderViolations(
+            this HipAccelerator accelerator,
+            AcceleratorStream stream,
+            int rows = 256)
+        {
+            using var mismatches = accelerator.Allocate1D<long>(1);
+            HipAlgorithmsException.ThrowIfFailed(
+                ilgpu_hip_selftest_lds_atomic_order(
+                    HipStream.PtrOf(stream),
+                    rows,
+                    (long*)mismatches.View.LoadEffectiveAddressAsPtr().ToPointer()),
+                nameof(rows));
+            stream.Synchronize();
+            return mismatches.GetAsArray1D()[0];
+        }
+
         /// <summary>CreateRadixSort (:1130-1337).</summary>
         public static RadixSort<T, TStride> CreateRadixSort<
             T,
@@ -159,7 +232,7 @@ namespace ILGPU.Algorithms.Hip
             where TRadixSortOperation : struct, IRadixSortOperation<TKey>
         {
             var (keyType, flags) = HipTypeMap.SortOperation<TKey, TRadixSortOperation>();
-            HipTypeMap.RequireIndexSequencer<TValue, TSequencer>();
+            int valueSource = HipTypeMap.ValueSource<TValue, TSequencer>();
             return (stream, keys, outputValues, sequencer, temp) =>
             {
                 long length = ValidLength(keys, nameof(keys));
@@ -179,7 +252,7 @@ namespace ILGPU.Algorithms.Hip
                         keyType,
                         sizeof(TValue),
                         flags,
-                        HipTypeMap.ValuesFromIndex,
+                        valueSource,
                         temp.LoadEffectiveAddressAsPtr().ToPointer(),
                         temp.Length * sizeof(int)),
                     nameof(temp));

@@ -65,7 +65,7 @@ namespace ILGPU.Algorithms.Hip
             HipRuntimeNativeMethods.Check(HipRuntimeNativeMethods.hipStreamSynchronize(StreamPtr));
 
         protected override ProfilingMarker AddProfilingMarkerInternal() =>
-            throw new NotSupportedException("profiling markers: use ilgpu_hip_profile_enable");
+            throw new NotSupportedException("profiling markers: use HipAccelerator.EnableKernelProfiling");
 
         protected override void DisposeAcceleratorObject(bool disposing)
         {
@@ -201,6 +201,30 @@ namespace ILGPU.Algorithms.Hip
 
         public void Synchronize() =>
             HipRuntimeNativeMethods.Check(HipRuntimeNativeMethods.hipDeviceSynchronize());
+
+        /// <summary>Version of the native library (major * 100 + minor).</summary>
+        public static int NativeLibraryVersion => HipAlgorithmsNativeMethods.ilgpu_hip_version();
+
+        /// <summary>Switches the library's per-kernel timing on or off (the counterpart
+        /// of ILGPU's ProfilingMarker, ProfilingMarker.cs:19-61): while it is on, every
+        /// kernel launch of the library is bracketed by a pair of HIP events on its
+        /// stream.  Process-wide; off by default.</summary>
+        public static void EnableKernelProfiling(bool enabled) =>
+            HipAlgorithmsException.ThrowIfFailed(
+                HipAlgorithmsNativeMethods.ilgpu_hip_profile_enable(enabled ? 1 : 0));
+
+        /// <summary>Launches and total milliseconds recorded for one kernel name
+        /// ("sort_onesweep", "scan", "reduce_partials", "histogram", ...) since the
+        /// last query of that name; waits for the recorded events.</summary>
+        public static (long Launches, double TotalMilliseconds) QueryKernelProfile(
+            string kernelName)
+        {
+            HipAlgorithmsException.ThrowIfFailed(
+                HipAlgorithmsNativeMethods.ilgpu_hip_profile_query(
+                    kernelName, out long launches, out double totalMs),
+                nameof(kernelName));
+            return (launches, totalMs);
+        }
 
         public void Dispose() => DefaultStream.Dispose();
     }

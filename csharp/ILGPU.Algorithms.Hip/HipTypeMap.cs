@@ -3,6 +3,7 @@
 // reference would JIT-compile) are NotSupportedException.
 using System;
 using System.Collections.Generic;
+using ILGPU.Algorithms.ComparisonOperations;
 using ILGPU.Algorithms.RadixSortOperations;
 using ILGPU.Algorithms.ScanReduceOperations;
 using ILGPU.Algorithms.Sequencers;
@@ -21,7 +22,10 @@ namespace ILGPU.Algorithms.Hip
         public const int ScanInclusive = 0, ScanExclusive = 1;
         // sort flags, value source
         public const int SortDescending = 1, SortFloatTotalOrder = 2;
-        public const int ValuesFromView = 0, ValuesFromIndex = 1;
+        public const int ValuesFromView = 0, ValuesFromIndex = 1, ValuesFromIndexAsFloat = 2;
+        // ilgpu_hip_transformer
+        public const int TransformConvert = 0, TransformNegate = 1, TransformBitComplement = 2,
+            TransformMultiply = 3;
         // histogram locators
         public const int LocatorIdentity = 0, LocatorModulo = 1;
 
@@ -105,23 +109,91 @@ namespace ILGPU.Algorithms.Hip
         public static int Kind(ScanKind kind) =>
             kind == ScanKind.Inclusive ? ScanInclusive : ScanExclusive;
 
-        // Identity sequencers: value = (T)index (Sequencer.cs:36-45, Sequencers.tt:25-37).
-        private static readonly HashSet<Type> IndexSequencers = new HashSet<Type>
+        // Identity sequencers: value = (T)index.  The integer ones truncate the
+        // index (Sequencer.cs:36-45, Sequencers.tt:25-37), Half/Float/DoubleSequencer
+        // convert it (Sequencer.cs:47-75).
+        private static readonly Dictionary<Type, int> IndexSequencers = new Dictionary<Type, int>
         {
-            typeof(IndexSequencer), typeof(Int32Sequencer), typeof(Int64Sequencer),
-            typeof(UInt32Sequencer), typeof(UInt64Sequencer),
+            { typeof(IndexSequencer), I32 },
+            { typeof(Int8Sequencer), I8 }, { typeof(Int16Sequencer), I16 },
+            { typeof(Int32Sequencer), I32 }, { typeof(Int64Sequencer), I64 },
+            { typeof(UInt8Sequencer), U8 }, { typeof(UInt16Sequencer), U16 },
+            { typeof(UInt32Sequencer), U32 }, { typeof(UInt64Sequencer), U64 },
+            { typeof(HalfSequencer), F16 }, { typeof(FloatSequencer), F32 },
+            { typeof(DoubleSequencer), F64 },
         };
 
-        /// <summary>True if the sequencer yields the element index.</summary>
-        public static void RequireIndexSequencer<TValue, TSequencer>()
+        /// <summary>The element type an identity sequencer produces; any other
+        /// sequencer (user code the reference would JIT-compile) is refused.</summary>
+        public static int IndexSequencer<TValue, TSequencer>()
             where TValue : unmanaged
             where TSequencer : struct, ISequencer<TValue>
         {
-            if (!IndexSequencers.Contains(typeof(TSequencer)))
+            if (!IndexSequencers.TryGetValue(typeof(TSequencer), out int type))
                 throw new NotSupportedException($"sequencer {typeof(TSequencer)}");
-            int size = System.Runtime.CompilerServices.Unsafe.SizeOf<TValue>();
-            if (size != 4 && size != 8)
-                throw new NotSupportedException("index values are 4 or 8 bytes wide");
+            if (type != ElementType<TValue>())
+                throw new NotSupportedException("sequencer and value type differ");
+            return type;
+        }
+
+        /// <summary>The value source of a key/value sort whose values an identity
+        /// sequencer generates.</summary>
+        public static int ValueSource<TValue, TSequencer>()
+            where TValue : unmanaged
+            where TSequencer : struct, ISequencer<TValue>
+        {
+            int type = IndexSequencer<TValue, TSequencer>();
+            return type == F16 || type == F32 || type == F64
+                ? ValuesFromIndexAsFloat
+                : ValuesFromIndex;
+        }
+
+        // Comparison* of ComparisonOperations.tt:26-45: first.CompareTo(second).
+        private static readonly Dictionary<Type, int> Comparisons =
+            new Dictionary<Type, int>
+        {
+            { typeof(ComparisonInt8), I8 },
+            { typeof(ComparisonInt16), I16 },
+            { typeof(ComparisonInt32), I32 },
+            { typeof(ComparisonInt64), I64 },
+            { typeof(ComparisonUInt8), U8 },
+            { typeof(ComparisonUInt16), U16 },
+            { typeof(ComparisonUInt32), U32 },
+            { typeof(ComparisonUInt64), U64 },
+            { typeof(ComparisonHalf), F16 },
+            { typeof(ComparisonFloat), F32 },
+            { typeof(ComparisonDouble), F64 },
+        };
+
+        /// <summary>Element type code of a comparison functor of the reference.</summary>
+        public static int ComparisonOperation<T, TComparisonOperation>()
+            where T : unmanaged
+            where TComparisonOperation : struct, IComparisonOperation<T>
+        {
+            if (!Comparisons.TryGetValue(typeof(TComparisonOperation), out int type))
+                throw new NotSupportedException(
+                    $"comparison operation {typeof(TComparisonOperation)}");
+            if (type != ElementType<T>())
+                throw new NotSupportedException("comparison operation and element type differ");
+            return type;
+        }
+
+        /// <summary>Transformer code and factor of a transformer of this layer's closed
+        /// set, or of the reference's IdentityTransformer (TransformExtensions.cs:42-55).
+        /// </summary>
+        public static (int Transformer, long Factor) Transformer<TSource, TTarget, TTransformer>(
+            TTransformer transformer)
+            where TSource : unmanaged
+            where TTarget : unmanaged
+            where TTransformer : struct, ITransformer<TSource, TTarget>
+        {
+            if (transformer is IHipTransformer known)
+                return (known.Code, known.Factor);
+            Type type = typeof(TTransformer);
+            if (type.IsGenericType &&
+                type.GetGenericTypeDefinition() == typeof(IdentityTransformer<>))
+                return (TransformConvert, 0);
+            throw new NotSupportedException($"transformer {type}");
         }
 
         /// <summary>Histogram locator code of a bin operation of this layer.</summary>

@@ -34,7 +34,7 @@ I8, I16, I32, I64, U8, U16, U32, U64, F16, F32, F64 = range(11)
 OP_ADD, OP_MAX, OP_MIN = 0, 1, 2
 SCAN_INCLUSIVE, SCAN_EXCLUSIVE = 0, 1
 SORT_DESCENDING, SORT_FLOAT_TOTAL_ORDER = 1, 2
-VALUES_FROM_VIEW, VALUES_FROM_INDEX = 0, 1
+VALUES_FROM_VIEW, VALUES_FROM_INDEX, VALUES_FROM_INDEX_AS_FLOAT = 0, 1, 2
 LOCATOR_IDENTITY, LOCATOR_MODULO = 0, 1
 (TRANSFORM_CONVERT, TRANSFORM_NEGATE, TRANSFORM_BIT_COMPLEMENT,
  TRANSFORM_MULTIPLY) = 0, 1, 2, 3
@@ -45,6 +45,7 @@ EXPORTS = [
     "ilgpu_hip_profile_query", "ilgpu_hip_radix_sort_temp_bytes",
     "ilgpu_hip_radix_sort_temp_bytes_strided",
     "ilgpu_hip_radix_sort_keys", "ilgpu_hip_radix_sort_pairs",
+    "ilgpu_hip_radix_sort_passes",
     "ilgpu_hip_selftest_lds_atomic_order", "ilgpu_hip_sort_check_device",
     "ilgpu_hip_sort_set_parameter",
     "ilgpu_hip_scan_temp_bytes", "ilgpu_hip_scan", "ilgpu_hip_scan_static",
@@ -132,6 +133,9 @@ def lib() -> ctypes.CDLL:
         L.ilgpu_hip_radix_sort_keys.argtypes = [vp, vp, i64, i64, i32, i32, vp, i64]
         L.ilgpu_hip_radix_sort_pairs.argtypes = [
             vp, vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, i64]
+        L.ilgpu_hip_radix_sort_passes.argtypes = [
+            vp, vp, i64, i64, i32, i32, ctypes.POINTER(i32), ctypes.POINTER(i32)]
+        L.ilgpu_hip_radix_sort_passes.restype = i32
         L.ilgpu_hip_selftest_lds_atomic_order.argtypes = [vp, i32, vp]
         L.ilgpu_hip_selftest_lds_atomic_order.restype = i32
         L.ilgpu_hip_sort_check_device.argtypes = [vp]
@@ -296,6 +300,9 @@ def radix_sort_pairs(keys: DeviceArray, values: DeviceArray,
                      temp: Optional[DeviceArray] = None, *,
                      descending: bool = False, float_total_order: bool = False,
                      values_from_index: bool = False, stream=None) -> None:
+    """values_from_index: the values are generated, value[i] = (TValue)i, as the
+    reference's sequencers do (integer value types: the index truncated; Half,
+    float and double values: the index converted)."""
     if temp is None:
         temp = temp_buffer(radix_sort_temp_bytes(
             keys.length, keys.dtype, values.dtype.itemsize, keys.stride,
@@ -309,8 +316,19 @@ def radix_sort_pairs(keys: DeviceArray, values: DeviceArray,
         _stream_ptr(stream), keys.ptr, keys.stride, values.ptr, values.stride,
         keys.length,
         keys.type_code, values.dtype.itemsize, flags,
-        VALUES_FROM_INDEX if values_from_index else VALUES_FROM_VIEW,
+        VALUES_FROM_VIEW if not values_from_index
+        else (VALUES_FROM_INDEX_AS_FLOAT if values.dtype.kind == "f" else VALUES_FROM_INDEX),
         temp.ptr, temp.nbytes))
+
+
+def radix_sort_passes(temp: DeviceArray, n: int, key_dtype, value_bytes: int = 0, *,
+                      stream=None):
+    """(executed, skipped) 8-bit passes of the last sort that used `temp`."""
+    executed, skipped = ctypes.c_int32(-1), ctypes.c_int32(-1)
+    check(lib().ilgpu_hip_radix_sort_passes(
+        _stream_ptr(stream), temp.ptr, temp.nbytes, n, type_code(key_dtype), value_bytes,
+        ctypes.byref(executed), ctypes.byref(skipped)))
+    return executed.value, skipped.value
 
 
 def selftest_lds_atomic_order(rows: int = 256, *, stream=None) -> int:

@@ -260,10 +260,13 @@ int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void* keys,
   if (flags & ~(ILGPU_HIP_SORT_DESCENDING | ILGPU_HIP_SORT_FLOAT_TOTAL_ORDER))
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   if (value_source != ILGPU_HIP_VALUES_FROM_VIEW &&
-      value_source != ILGPU_HIP_VALUES_FROM_INDEX)
+      value_source != ILGPU_HIP_VALUES_FROM_INDEX &&
+      value_source != ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT)
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
-  if (value_source == ILGPU_HIP_VALUES_FROM_INDEX && value_bytes != 4 &&
-      value_bytes != 8)
+  if (value_source == ILGPU_HIP_VALUES_FROM_INDEX && value_bytes == 16)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT && value_bytes != 2 &&
+      value_bytes != 4 && value_bytes != 8)
     return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   const int32_t rc = check_temp(
       temp, temp_bytes,
@@ -281,6 +284,24 @@ int32_t ilgpu_hip_selftest_lds_atomic_order(ilgpu_hip_stream_t stream,
   if (!aligned_to(mismatches, 8)) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
   return launch_lds_atomic_order_selftest(static_cast<hipStream_t>(stream), rows,
                                           mismatches);
+}
+
+int32_t ilgpu_hip_radix_sort_passes(ilgpu_hip_stream_t stream, const void* temp,
+                                    int64_t temp_bytes, int64_t n, int32_t key_type,
+                                    int32_t value_bytes, int32_t* executed,
+                                    int32_t* skipped) {
+  if (executed == nullptr || skipped == nullptr) return ILGPU_HIP_ERROR_NULL_VIEW;
+  const int kb = elem_size(key_type);
+  if (kb < 0) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (value_bytes != 0 && value_bytes != 1 && value_bytes != 2 && value_bytes != 4 &&
+      value_bytes != 8 && value_bytes != 16)
+    return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  if (n < 1) return ILGPU_HIP_ERROR_OUT_OF_RANGE;
+  if (n > radix_sort_max_length()) return ILGPU_HIP_ERROR_NOT_SUPPORTED;
+  const int32_t rc = check_temp(temp, temp_bytes, radix_sort_temp_bytes(n, kb, value_bytes));
+  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  return read_sort_plan(static_cast<hipStream_t>(stream), temp, n, kb, value_bytes, executed,
+                        skipped);
 }
 
 int32_t ilgpu_hip_sort_check_device(ilgpu_hip_stream_t stream) {

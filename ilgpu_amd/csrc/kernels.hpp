@@ -61,6 +61,10 @@ int32_t launch_lds_atomic_order_selftest(hipStream_t stream, int rows, int64_t* 
 // `stream` is being captured and the device has not been asked yet).  Every
 // sort calls it first.
 int32_t check_sort_device(hipStream_t stream);
+// How many passes the last sort that used `temp` (same n, key size, value size,
+// dense views) ran, and how many it found unnecessary; waits for the stream.
+int32_t read_sort_plan(hipStream_t stream, const void* temp, int64_t n, int key_bytes,
+                       int value_bytes, int32_t* executed, int32_t* skipped);
 
 // scan.hip: Unique (consecutive duplicates removed in place, new length to
 // out_length[0] on the device).

@@ -189,6 +189,26 @@ int32_t check_sort_device(hipStream_t stream) {
   return mismatches == 0 ? ILGPU_HIP_SUCCESS : ILGPU_HIP_ERROR_NOT_SUPPORTED;
 }
 
+int32_t read_sort_plan(hipStream_t stream, const void* temp, int64_t n, int key_bytes,
+                       int value_bytes, int32_t* executed, int32_t* skipped) {
+  // Inputs of one tile are sorted by one block without a plan: every pass runs.
+  if (n <= (int64_t)tile_keys(key_bytes, value_bytes, kSortBlock) &&
+      g_sort_small_kernel.load(std::memory_order_relaxed) != 0) {
+    *executed = key_bytes;
+    *skipped = 0;
+    return ILGPU_HIP_SUCCESS;
+  }
+  const TempLayout L = make_layout(n, key_bytes, value_bytes);
+  const char* base = reinterpret_cast<const char*>(align_up((int64_t)(uintptr_t)temp, 256));
+  SortPlan plan;
+  ILGPU_HIP_CHECK(hipMemcpyAsync(&plan, base + L.plan, sizeof(plan), hipMemcpyDeviceToHost,
+                                 stream));
+  ILGPU_HIP_CHECK(hipStreamSynchronize(stream));
+  *executed = (int32_t)plan.executed;
+  *skipped = key_bytes - (int32_t)plan.executed;
+  return ILGPU_HIP_SUCCESS;
+}
+
 int64_t radix_sort_max_length() { return kMaxSortLength; }
 
 int64_t radix_sort_temp_bytes(int64_t n, int key_bytes, int value_bytes,

@@ -41,6 +41,8 @@
 // unit that launches it, hence a header and not a library of kernels.)
 #pragma once
 
+#include <hip/hip_fp16.h>
+
 #include <atomic>
 #include <type_traits>
 
@@ -162,6 +164,30 @@ template <> struct ValueOf<2> { using type = uint16_t; };
 template <> struct ValueOf<4> { using type = uint32_t; };
 template <> struct ValueOf<8> { using type = uint64_t; };
 template <> struct ValueOf<16> { using type = Bytes16; };
+
+// The value a sequencer gives element i (Sequencers.tt:25-37, Sequencer.cs:36-75):
+// mode 1 = the integer sequencers and IndexSequencer, (T)i with T as wide as the
+// value; mode 2 = HalfSequencer, FloatSequencer and DoubleSequencer, (T)i in
+// floating point (long to float rounds to nearest even, Half goes through
+// float as the C# conversion does).
+template <int VALUE_BYTES>
+__device__ __forceinline__ typename ValueOf<VALUE_BYTES>::type index_value(int64_t i, int mode) {
+  using Val = typename ValueOf<VALUE_BYTES>::type;
+  if constexpr (VALUE_BYTES == 1) {
+    return (Val)(uint8_t)i;
+  } else if constexpr (VALUE_BYTES == 2) {
+    if (mode == 2) return (Val)__half_as_ushort(__float2half((float)i));
+    return (Val)(uint16_t)i;
+  } else if constexpr (VALUE_BYTES == 4) {
+    if (mode == 2) return (Val)__float_as_uint((float)i);
+    return (Val)(uint32_t)i;
+  } else if constexpr (VALUE_BYTES == 8) {
+    if (mode == 2) return (Val)(uint64_t)__double_as_longlong((double)i);
+    return (Val)(uint64_t)i;
+  } else {
+    return Val{};  // 16-byte values are never generated (refused by the entry point)
+  }
+}
 
 // Keys per thread and tile.  Long tiles pay: the runs they scatter are longer
 // (fewer partial cache lines) and there are fewer tiles to chain.  Keys-only
@@ -445,7 +471,7 @@ __device__ __forceinline__ void sort_tile(
     const typename ValueOf<VALUE_BYTES>::type* __restrict__ src_vals,
     typename ValueOf<VALUE_BYTES>::type* __restrict__ dst_vals,
     int64_t tile_base, int valid, int tile, int pass, const KeyXform& xf,
-    const uint32_t* __restrict__ excl, uint32_t* status, bool make_index,
+    const uint32_t* __restrict__ excl, uint32_t* status, int make_index,
     unsigned char* s_stage, uint32_t* s_global_off, uint32_t* s_scan,
     const uint32_t (&hot)[kMaxHot], uint32_t spin_limit, bool in_raw, bool out_raw) {
   using K = typename KeyOf<KEY_BYTES>::type;
@@ -504,8 +530,7 @@ __device__ __forceinline__ void sort_tile(
       const int local = first_local + j * kSubLanes;
       if (FULL || local < valid) {
         if (make_index) {
-          if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)(tile_base + local);
-          else if constexpr (VALUE_BYTES == 8) val[j] = (Val)(uint64_t)(tile_base + local);
+          val[j] = index_value<VALUE_BYTES>(tile_base + local, make_index);
         } else {
           val[j] = src_vals[tile_base + local];
         }
@@ -786,8 +811,9 @@ void onesweep_kernel(
   K* dst_keys = src_alt ? keys_a : keys_b;
   const Val* src_vals = src_alt ? vals_b : vals_a;
   Val* dst_vals = src_alt ? vals_a : vals_b;
-  const bool make_index = VALUE_BYTES > 0 && values_from_index &&
-                          plan->first_executed == (uint32_t)pass;
+  // 0, or the kind of index values the first pass that runs generates
+  const int make_index =
+      VALUE_BYTES > 0 && plan->first_executed == (uint32_t)pass ? values_from_index : 0;
   const bool in_raw = plan->first_executed == (uint32_t)pass;
   const bool out_raw = plan->last_executed == (uint32_t)pass;
   const int tid = threadIdx.x;
@@ -1585,8 +1611,7 @@ void small_sort_kernel(typename KeyOf<KEY_BYTES>::type* keys,
       if constexpr (FLOAT_KEYS) key[j] = ordered_bits(key[j], xf);
       if constexpr (kPairs) {
         if (values_from_index) {
-          if constexpr (VALUE_BYTES == 4) val[j] = (Val)(uint32_t)local;
-          else if constexpr (VALUE_BYTES == 8) val[j] = (Val)(uint64_t)local;
+          val[j] = index_value<VALUE_BYTES>(local, values_from_index);
         } else {
           val[j] = vals[local];
         }
@@ -1694,7 +1719,6 @@ __global__ __launch_bounds__(256) void finish_kernel(
     typename ValueOf<VALUE_BYTES>::type* vals_a,
     const typename ValueOf<VALUE_BYTES>::type* vals_b, int64_t n,
     const SortPlan* __restrict__ plan, int values_from_index) {
-  using Val = typename ValueOf<VALUE_BYTES>::type;
   const bool copy_back = plan->final_in_alt != 0;
   const bool fill_index =
       VALUE_BYTES > 0 && values_from_index && plan->executed == 0;
@@ -1706,8 +1730,7 @@ __global__ __launch_bounds__(256) void finish_kernel(
       keys_a[i] = keys_b[i];
       if constexpr (VALUE_BYTES > 0) vals_a[i] = vals_b[i];
     } else {
-      if constexpr (VALUE_BYTES == 4) vals_a[i] = (Val)(uint32_t)i;
-      else if constexpr (VALUE_BYTES == 8) vals_a[i] = (Val)(uint64_t)i;
+      if constexpr (VALUE_BYTES > 0) vals_a[i] = index_value<VALUE_BYTES>(i, values_from_index);
     }
   }
 }
@@ -1783,7 +1806,9 @@ int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L
   SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
   uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
   const int passes = KEY_BYTES;
-  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
+  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX
+                             ? 1
+                             : (a.value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT ? 2 : 0);
   const bool float_keys = (xf.reference_term | xf.total_term) != 0;
   auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false, BLOCK>;
   if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
@@ -1881,7 +1906,9 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
     ProfileScope scope(stream, "sort_small");
     hipLaunchKernelGGL(kernel, dim3(1), dim3(kSortBlock), 0, stream, static_cast<K*>(a.keys),
                        static_cast<Val*>(a.values), (int)a.n, xf,
-                       a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0);
+                       a.value_source == ILGPU_HIP_VALUES_FROM_INDEX
+                             ? 1
+                             : (a.value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT ? 2 : 0));
     ILGPU_HIP_CHECK(hipGetLastError());
     return ILGPU_HIP_SUCCESS;
   }
@@ -1911,7 +1938,9 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
   uint32_t* hist = reinterpret_cast<uint32_t*>(base + L.hist);
   const int passes = KEY_BYTES;
-  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX ? 1 : 0;
+  const int from_index = a.value_source == ILGPU_HIP_VALUES_FROM_INDEX
+                             ? 1
+                             : (a.value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT ? 2 : 0);
 
   int32_t rc = launch_zero_words(stream, hist, (L.total - L.zero_begin) / 4);
   if (rc != ILGPU_HIP_SUCCESS) return rc;

@@ -481,7 +481,10 @@ CreateRadixSortPairsWithSequencer(Accelerator&) {
             TypeCode<TKey>::value,
             (int32_t)sizeof(TValue),
             TRadixSortOperation::Descending ? ILGPU_HIP_SORT_DESCENDING : 0,
-            ILGPU_HIP_VALUES_FROM_INDEX, tempView.LoadEffectiveAddressAsPtr(),
+            // Half/Float/DoubleSequencer convert the index, the others truncate it
+            std::is_floating_point<TValue>::value ? ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT
+                                                  : ILGPU_HIP_VALUES_FROM_INDEX,
+            tempView.LoadEffectiveAddressAsPtr(),
             tempView.Length() * 4),
         "tempView");
   };

@@ -97,11 +97,17 @@ enum {
 
 /* Where the values of a key/value sort come from: the values view itself
  * (ViewSourceSequencer, Sequencer.cs:79-102) or value[i] = (TValue)i computed
- * on the fly (IndexSequencer / Int32Sequencer ... , Sequencer.cs:36-45,
- * Sequencers.tt:25-37; integer value types of 4 or 8 bytes). */
+ * on the fly.  FROM_INDEX: TValue is the integer type as wide as the value
+ * (IndexSequencer, Sequencer.cs:36-45, and Int8Sequencer .. UInt64Sequencer,
+ * Sequencers.tt:25-37: the index truncated to 1, 2, 4 or 8 bytes).
+ * FROM_INDEX_AS_FLOAT: TValue is the floating-point type as wide as the value
+ * (HalfSequencer, FloatSequencer, DoubleSequencer, Sequencer.cs:47-75: 2, 4 or
+ * 8 bytes; long to float rounds to nearest even, Half goes through float as
+ * the C# conversion does, so indices from 65520 on give +infinity). */
 typedef enum ilgpu_hip_value_source {
   ILGPU_HIP_VALUES_FROM_VIEW = 0,
-  ILGPU_HIP_VALUES_FROM_INDEX = 1
+  ILGPU_HIP_VALUES_FROM_INDEX = 1,
+  ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT = 2
 } ilgpu_hip_value_source;
 
 /* Histogram bin locators (IComputeSingleBinOperation, IHistogramOperations.cs:
@@ -167,14 +173,26 @@ int32_t ilgpu_hip_radix_sort_keys(ilgpu_hip_stream_t stream, void *keys,
                                   int32_t flags, void *temp,
                                   int64_t temp_bytes);
 
-/* value_bytes in {1, 2, 4, 8, 16}.  With ILGPU_HIP_VALUES_FROM_INDEX the
- * incoming contents of `values` are ignored and value_bytes must be 4 or 8. */
+/* value_bytes in {1, 2, 4, 8, 16}.  With ILGPU_HIP_VALUES_FROM_INDEX (value_bytes
+ * 1, 2, 4 or 8) and ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT (2, 4 or 8) the incoming
+ * contents of `values` are ignored. */
 int32_t ilgpu_hip_radix_sort_pairs(ilgpu_hip_stream_t stream, void *keys,
                                    int64_t key_stride, void *values,
                                    int64_t value_stride, int64_t n,
                                    int32_t key_type, int32_t value_bytes,
                                    int32_t flags, int32_t value_source,
                                    void *temp, int64_t temp_bytes);
+
+/* How many 8-bit passes the last sort that used `temp` ran and how many it
+ * found unnecessary (a pass whose digit is the same for every key is skipped:
+ * keys below 2^16 run two passes of four, equal keys none).  Same n, key_type
+ * and value_bytes (0 for keys only) as that sort, dense views; waits for
+ * `stream`.  The reference runs all NumBits / 2 passes whatever the keys
+ * (RadixSortExtensions.cs:1276-1334) and has nothing to report. */
+int32_t ilgpu_hip_radix_sort_passes(ilgpu_hip_stream_t stream, const void *temp,
+                                    int64_t temp_bytes, int64_t n,
+                                    int32_t key_type, int32_t value_bytes,
+                                    int32_t *executed, int32_t *skipped);
 
 /* Device self-check of the one hardware property the sort's ranking relies
  * on beyond the programming model: the lanes of ONE returning LDS atomic
@@ -306,6 +324,11 @@ int32_t ilgpu_hip_reduce(ilgpu_hip_stream_t stream, const void *in,
  * bin type's MaxValue (an increment found the bin holding MaxValue,
  * HistogramOperations.tt:36-40); NULL selects the unchecked variant.
  * in_type: any ilgpu_hip_type except F16.
+ * Floating-point bins must live in ordinary device memory (hipMalloc: coarse
+ * grained).  With more bins than LDS holds their single increments go through
+ * the hardware's floating-point atomic add in L2, which is exact there; for
+ * fine-grained, host-mapped or managed memory the hardware does not promise
+ * that, and no reference fixture covers floating-point bins at all.
  */
 int32_t ilgpu_hip_histogram(ilgpu_hip_stream_t stream, const void *in,
                             int64_t n, int64_t stride, int32_t in_type,

@@ -34,6 +34,16 @@ def test_source_digest_ignores_comments_and_layout_but_not_code(tmp_path, monkey
     (tmp_path / "c.hip").write_text("int f() {\n  return 2;\n}\n")
     assert bench.source_digest("a.hip") == bench.source_digest("b.hip")
     assert bench.source_digest("a.hip") != bench.source_digest("c.hip")
+    # the shared headers and the compiler flags count too
+    before = bench.source_digest("a.hip")
+    (tmp_path / "common.hpp").write_text("constexpr int kWaveSize = 64;\n")
+    with_header = bench.source_digest("a.hip")
+    assert with_header != before
+    (tmp_path / "common.hpp").write_text("constexpr int kWaveSize = 64;  // a wave\n")
+    assert bench.source_digest("a.hip") == with_header
+    from ilgpu_amd import build
+    monkeypatch.setattr(build, "FLAGS", build.FLAGS + ["-DX"])
+    assert bench.source_digest("a.hip") != with_header
 
 
 def test_stale_counters_are_not_reported_as_traffic(tmp_path, monkeypatch):

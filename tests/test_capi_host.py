@@ -96,7 +96,9 @@ def test_sort_argument_validation():
     # pairs
     assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, None, 1, 16, capi.U32, 4, 0, 0, FAKE, big) == capi.ERROR_NULL_VIEW
     assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 3, 0, 0, FAKE, big) == capi.ERROR_NOT_SUPPORTED
-    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 2, 0, capi.VALUES_FROM_INDEX, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 16, 0, capi.VALUES_FROM_INDEX, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 1, 0, capi.VALUES_FROM_INDEX_AS_FLOAT, FAKE, big) == capi.ERROR_NOT_SUPPORTED
+    assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 4, 0, 3, FAKE, big) == capi.ERROR_NOT_SUPPORTED
     assert L.ilgpu_hip_radix_sort_pairs(None, FAKE, 1, FAKE, 1, 16, capi.U32, 4, 0, 0, FAKE, 64) == capi.ERROR_OUT_OF_RANGE
 
 

@@ -165,3 +165,42 @@ def test_public_surface_names_the_references_methods():
     has("HipReductionExtensions.cs", "CreateReduction", "Reduce", "ReduceAsync")
     has("HipHistogramExtensions.cs", "CreateHistogram", "CreateHistogramUnchecked", "Histogram",
         "HistogramUnchecked")
+
+
+def test_every_import_is_used_by_the_layers_public_surface():
+    # A DllImport nobody calls is an entry point C# users cannot reach.  The one
+    # exception is deliberate: ilgpu_hip_sort_set_parameter is a process-wide
+    # test hook of the library and stays out of the public surface.
+    hidden = {"ilgpu_hip_sort_set_parameter"}
+    others = ""
+    for name in sorted(os.listdir(CSHARP)):
+        if name.endswith(".cs") and name != "HipAlgorithmsNativeMethods.cs":
+            others += strip_comments(open(os.path.join(CSHARP, name)).read())
+    for name in csharp_prototypes():
+        used = re.search(r"\b" + name + r"\s*\(", others) is not None
+        assert used != (name in hidden), name
+
+
+def test_reference_surface_of_the_neighbouring_primitives_is_there():
+    # Unique, Initialize, Sequence, Reorder and Transform: every public method of
+    # the reference's extension classes has a counterpart of the same name.
+    expected = {
+        "HipUniqueExtensions.cs": ["ComputeUniqueTempStorageSize", "CreateUnique", "Unique"],
+        "HipInitializeExtensions.cs": ["CreateInitializer", "Initialize"],
+        "HipSequenceExtensions.cs": ["CreateSequencer", "CreateBatchedSequencer",
+                                     "CreateRepeatedSequencer", "CreateRepeatedBatchedSequencer",
+                                     "Sequence", "RepeatedSequence", "BatchedSequence",
+                                     "RepeatedBatchedSequence"],
+        "HipReorderExtensions.cs": ["CreateReorderTransformer", "Reorder", "ReorderTransform"],
+        "HipTransformExtensions.cs": ["CreateTransformer", "Transform"],
+    }
+    for file_name, methods in expected.items():
+        text = strip_comments(open(os.path.join(CSHARP, file_name)).read())
+        for method in methods:
+            assert re.search(r"public\s+static\s+[^;{(]*\b" + method + r"\s*<", text, flags=re.S), \
+                (file_name, method)
+    type_map = open(os.path.join(CSHARP, "HipTypeMap.cs")).read()
+    for functor in ["ComparisonInt8", "ComparisonUInt64", "ComparisonHalf", "ComparisonDouble",
+                    "Int8Sequencer", "UInt16Sequencer", "HalfSequencer", "FloatSequencer",
+                    "DoubleSequencer", "IdentityTransformer"]:
+        assert functor in type_map, functor

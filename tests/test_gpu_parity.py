@@ -517,20 +517,47 @@ def test_sort_pairs_16_byte_values():
     assert np.array_equal(got, values[perm])
 
 
-@pytest.mark.parametrize("value_dtype", [np.uint32, np.int64])
+@pytest.mark.parametrize("value_dtype", [np.uint32, np.int64, np.int8, np.uint8, np.int16,
+                                         np.uint16, np.float16, np.float32, np.float64])
 def test_sort_pairs_values_from_index(value_dtype):
-    # Sequencer form (RadixSortExtensions.cs:1017-1074 with Int32Sequencer /
-    # Int64Sequencer): value[i] = i, whatever the values view held before.
+    # Sequencer form (RadixSortExtensions.cs:1017-1074): value[i] = (TValue)i,
+    # whatever the values view held before.  Integer sequencers truncate the index
+    # (Sequencers.tt:25-37); HalfSequencer, FloatSequencer and DoubleSequencer
+    # convert it (Sequencer.cs:47-75: Half through float, so +inf from 65520 on).
+    def sequencer(index):
+        if np.dtype(value_dtype) == np.float16:
+            return index.astype(np.float32).astype(np.float16)
+        return index.astype(value_dtype)           # numpy truncates integers as C# does
+
     for keys in (datagen.uniform_u64(100003), datagen.constant_u32(5000),
-                 datagen.uniform_u32(9000) & np.uint32(0xFF)):
+                 datagen.uniform_u32(9000) & np.uint32(0xFF),
+                 datagen.uniform_u32(18432 * 3 + 5)):          # several tiles: the passes
         n = keys.size
         dk = D.from_numpy(keys)
         dv = D.from_numpy(np.full(n, 99, dtype=value_dtype))
+        with np.errstate(over="ignore"):
+            expect = sequencer(np.argsort(keys, kind="stable"))
         capi.radix_sort_pairs(dk, dv, values_from_index=True)
         sync()
-        perm = np.argsort(keys, kind="stable")
-        assert np.array_equal(dk.numpy(), keys[perm])
-        assert np.array_equal(dv.numpy(), perm.astype(value_dtype))
+        assert np.array_equal(dk.numpy(), np.sort(keys, kind="stable"))
+        assert bits_equal(dv.numpy(), expect), np.dtype(value_dtype).name
+    # hand-evaluated: index 2049 is not a Half (rounds to even: 2048), 65519 rounds
+    # to 65504, 65520 to infinity; 16777217 is not a float (rounds to 16777216)
+    if np.dtype(value_dtype) == np.float16:
+        n = 70000
+        dk, dv = D.from_numpy(np.arange(n, dtype=np.uint32)), D.zeros(n, np.float16)
+        capi.radix_sort_pairs(dk, dv, values_from_index=True)
+        sync()
+        got = dv.numpy().view(np.uint16)
+        assert got[2049] == 0x6800 and got[2051] == 0x6802       # 2048, 2052
+        assert got[65519] == 0x7BFF and got[65520] == 0x7C00     # 65504, +inf
+    if np.dtype(value_dtype) == np.float32:
+        n = (1 << 24) + 4
+        dk, dv = D.from_numpy(np.arange(n, dtype=np.uint32)), D.zeros(n, np.float32)
+        capi.radix_sort_pairs(dk, dv, values_from_index=True)
+        sync()
+        got = dv.numpy()
+        assert got[16777217] == 16777216.0 and got[16777219] == 16777220.0
 
 
 def test_sort_reuses_dirty_temp_and_unaligned_key_view():
