@@ -4,7 +4,15 @@
 (in parallel) and links them into ``ilgpu_amd/lib/libilgpu_hip_algorithms.so``.
 hipcc cross-compiles, so no GPU is needed.  The shared library is kept in the
 tree (git-ignored) so that it travels with the source to the machine that runs
-it.
+it.  The same call builds the C++ host-layer test program and the
+micro-benchmarks of ``bench_bounds.hip``.
+
+``python -m ilgpu_amd.build --variant NAME -D MACRO=VALUE [-D ...] [--units a,b]``
+builds ``ilgpu_amd/lib/variants/libNAME.so``: the named units (default: all)
+recompiled with the given tuning macros, the rest taken from the last full
+build.  ``ILGPU_HIP_ALGORITHMS_LIB=<that file>`` makes ``ilgpu_amd.capi``, and
+with it ``bench.py`` and the tests, load the variant: this is how the measured
+alternatives quoted in the kernels' comments were timed.
 """
 from __future__ import annotations
 
@@ -36,9 +44,9 @@ def sources() -> list[str]:
         os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+def _compile(src: str, obj_dir: str = OBJ_DIR, defines: tuple[str, ...] = ()) -> str:
+    obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
+    cmd = [HIPCC, *FLAGS, *(f"-D{d}" for d in defines), "-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
@@ -62,6 +70,48 @@ def build(jobs: int | None = None) -> str:
     return LIB_PATH
 
 
+def build_variant(name: str, defines: list[str], units: list[str] | None = None) -> str:
+    """Links a library whose `units` (file names in csrc/ without .hip; all of
+    them when None) are compiled with -D<define> for every entry of `defines`;
+    the other units come from the objects of the last full build."""
+    all_sources = sources()
+    chosen = [s for s in all_sources
+              if units is None or os.path.basename(s)[:-4] in units]
+    if units is not None and len(chosen) != len(units):
+        raise ValueError(f"unknown unit in {units}")
+    var_dir = os.path.join(LIB_DIR, "variants")
+    obj_dir = os.path.join(var_dir, "obj_" + name)
+    os.makedirs(obj_dir, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        new = list(pool.map(lambda s: _compile(s, obj_dir, tuple(defines)), chosen))
+    kept = [os.path.join(OBJ_DIR, os.path.basename(s)[:-4] + ".o")
+            for s in all_sources if s not in chosen]
+    missing = [o for o in kept if not os.path.exists(o)]
+    if missing:
+        raise RuntimeError(f"run a full build first: {missing[0]} is missing")
+    out = os.path.join(var_dir, f"lib{name}.so")
+    proc = subprocess.run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out,
+                           *new, *kept], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    return out
+
+
+BOUNDS_SRC = os.path.join(os.path.dirname(HERE), "bench_bounds.hip")
+BOUNDS_BIN = os.path.join(LIB_DIR, "bench_bounds")
+
+
+def build_bounds() -> str:
+    """Compiles the micro-benchmarks that bound the kernels (a program of its
+    own: it does not link the library)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [HIPCC, *FLAGS, BOUNDS_SRC, "-o", BOUNDS_BIN]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"bench_bounds build failed:\n{proc.stderr}")
+    return BOUNDS_BIN
+
+
 HOST_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp",
                              "host_api_tests.cpp")
 HOST_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp",
@@ -82,5 +132,16 @@ def build_host_example() -> str:
 
 
 if __name__ == "__main__":
-    print(build())
-    print(build_host_example())
+    import argparse
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--variant", help="name of a tuning variant to build instead of the library")
+    ap.add_argument("-D", dest="defines", action="append", default=[], metavar="MACRO=VALUE")
+    ap.add_argument("--units", help="comma-separated csrc units the macros apply to (default: all)")
+    cli = ap.parse_args()
+    if cli.variant:
+        print(build_variant(cli.variant, cli.defines,
+                            cli.units.split(",") if cli.units else None))
+    else:
+        print(build())
+        print(build_host_example())
+        print(build_bounds())

@@ -127,7 +127,20 @@ constexpr int kLargeMinTilesPerCuPairs = 2;
 // Lanes that rank together (a sub-tile row): one wave.
 constexpr int kSubLanes = kWaveSize;
 constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
-constexpr int kHistBlock = 512;
+#ifndef ILGPU_HIP_SORT_HIST_BLOCK
+#define ILGPU_HIP_SORT_HIST_BLOCK 512
+#endif
+#ifndef ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU
+#define ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU 2
+#endif
+#ifndef ILGPU_HIP_SORT_HIST_NT
+#define ILGPU_HIP_SORT_HIST_NT 1
+#endif
+#ifndef ILGPU_HIP_SORT_HIST_UNROLL
+#define ILGPU_HIP_SORT_HIST_UNROLL 2
+#endif
+constexpr int kHistUnroll = ILGPU_HIP_SORT_HIST_UNROLL;
+constexpr int kHistBlock = ILGPU_HIP_SORT_HIST_BLOCK;
 #ifndef ILGPU_HIP_SORT_HIST_LDS_WORDS
 #define ILGPU_HIP_SORT_HIST_LDS_WORDS 16384
 #endif
@@ -293,6 +306,14 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  // Non-temporal loads: 0.180 against 0.217 ms for 2^28 u32 keys.  The kernel
+  // is bound by the rate of LDS instructions (a wave's atomic takes the LDS of
+  // a compute unit about five cycles whatever its addresses) next to the key
+  // stream, and the two overlap better when the keys do not allocate in L2.
+  // Two vectors per round: one is 0.235 ms, four 0.208.
+  auto load_keys = [](const V* p) -> V {
+    return ILGPU_HIP_SORT_HIST_NT ? __builtin_nontemporal_load(p) : *p;
+  };
   const uintptr_t addr = reinterpret_cast<uintptr_t>(keys);
   int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(K));
   if (head > n) head = n;
@@ -301,16 +322,18 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
   const int64_t tail_start = head + nvec * VN;
   const int64_t stride = (int64_t)gridDim.x * kHistBlock;
   int64_t i = (int64_t)blockIdx.x * kHistBlock + threadIdx.x;
-  for (; i + stride < nvec; i += 2 * stride) {
-    V a = body[i];
-    V b = body[i + stride];
+  for (; i + (kHistUnroll - 1) * stride < nvec; i += kHistUnroll * stride) {
+    V v[kHistUnroll];
 #pragma unroll
-    for (int k = 0; k < VN; ++k) count(a[k]);
+    for (int u = 0; u < kHistUnroll; ++u) v[u] = load_keys(&body[i + u * stride]);
 #pragma unroll
-    for (int k = 0; k < VN; ++k) count(b[k]);
+    for (int u = 0; u < kHistUnroll; ++u) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) count(v[u][k]);
+    }
   }
   for (; i < nvec; i += stride) {
-    V a = body[i];
+    V a = load_keys(&body[i]);
 #pragma unroll
     for (int k = 0; k < VN; ++k) count(a[k]);
   }
@@ -433,6 +456,16 @@ template <int KEY_BYTES, int VALUE_BYTES, int BLOCK> struct SortTile {
       kValueStageBytes > kKeyOrCounterBytes ? kValueStageBytes : kKeyOrCounterBytes;
 };
 
+// Cache policy of a pass's key loads and scattered stores.  Measured on 2^28
+// u32 keys, ms per pass: plain / plain 0.477, non-temporal loads 0.486,
+// non-temporal stores 0.658 (the scattered stores rely on L2 to merge the
+// pieces of a line that different waves write).
+#ifndef ILGPU_HIP_SORT_NT_LOAD
+#define ILGPU_HIP_SORT_NT_LOAD 0
+#endif
+#ifndef ILGPU_HIP_SORT_NT_STORE
+#define ILGPU_HIP_SORT_NT_STORE 0
+#endif
 template <int KEY_BYTES, int ITEMS, bool FULL>
 __device__ __forceinline__ void load_tile_keys(
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src, int64_t tile_base,
@@ -441,7 +474,9 @@ __device__ __forceinline__ void load_tile_keys(
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
     const int local = first_local + j * kSubLanes;
-    if (FULL || local < valid) key[j] = src[tile_base + local];
+    if (FULL || local < valid)
+      key[j] = ILGPU_HIP_SORT_NT_LOAD ? __builtin_nontemporal_load(&src[tile_base + local])
+                                      : src[tile_base + local];
     else key[j] = 0;
   }
 }
@@ -1444,7 +1479,8 @@ void onesweep_pipelined_kernel(
       if (kFull || i < valid) {
         const K k = s_keys[i];
         const uint32_t g = global_off[digit(k)] + (uint32_t)i;
-        dst_keys[g] = k;
+        if (ILGPU_HIP_SORT_NT_STORE) __builtin_nontemporal_store(k, &dst_keys[g]);
+        else dst_keys[g] = k;
       }
       if (j % ILGPU_HIP_SORT_WRITE_GROUP == ILGPU_HIP_SORT_WRITE_GROUP - 1)
         __builtin_amdgcn_sched_barrier(0);
@@ -1868,6 +1904,8 @@ int32_t launch_passes_pipelined(hipStream_t stream, const SortArgs& a, const Tem
   int64_t grid = cus;  // 1024 threads and 150 KiB of LDS: one block per compute unit
   if (grid > L.tiles) grid = L.tiles;
   const int groups = grid < kTicketGroups ? (int)grid : kTicketGroups;
+  // Chunks of 16 and 32 tiles, which the write pattern by itself prefers
+  // (bench_bounds scatter), lose here: 0.492 and 0.572 ms per pass against 0.484.
   int chunk_shift = 0;
   while (chunk_shift < kMaxChunkShift && (grid << (chunk_shift + 1)) <= L.tiles) ++chunk_shift;
   const uint32_t spin_limit = g_sort_spin_limit.load(std::memory_order_relaxed);
@@ -1953,7 +1991,8 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
     const size_t lds = (size_t)((passes * kRadix) << shift) * 4;
     int64_t blocks = div_up(div_up(a.n, Vec16<K>::N), kHistBlock);
     // Two blocks of 64 KiB of counters are resident per CU: no second round.
-    if (blocks > (int64_t)cus * 2) blocks = (int64_t)cus * 2;
+    if (blocks > (int64_t)cus * ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU)
+      blocks = (int64_t)cus * ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU;
     if (blocks < 1) blocks = 1;
     ProfileScope scope(stream, "sort_histogram");
     auto* histogram_kernel = sort_histogram_kernel<K, false>;

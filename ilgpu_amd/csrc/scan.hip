@@ -39,6 +39,15 @@ namespace {
 #ifndef ILGPU_HIP_SCAN_VECS
 #define ILGPU_HIP_SCAN_VECS 16
 #endif
+#ifndef ILGPU_HIP_SCAN_WAVES_PER_EU
+#define ILGPU_HIP_SCAN_WAVES_PER_EU 4
+#endif
+#ifndef ILGPU_HIP_SCAN_NT_LOAD
+#define ILGPU_HIP_SCAN_NT_LOAD 1
+#endif
+#ifndef ILGPU_HIP_SCAN_NT_STORE
+#define ILGPU_HIP_SCAN_NT_STORE 1
+#endif
 // 8-byte status words per tile: one 128-byte line each.  Every resident block
 // polls the words of the few dozen tiles before it with loads that go past the
 // L2; packed eight bytes apart those words share a handful of lines, and the
@@ -264,7 +273,7 @@ __device__ __forceinline__ T resolve_prefix(const TileState<T>& st, int tile,
 // the compiler takes 180 to 256 registers for the floating-point Max and Min
 // kernels, which halves their residency (measured 0.56 -> 0.44 ms at 2^28 float).
 template <typename T, int OP, bool VECTOR>
-__global__ __launch_bounds__(kBlock, 4) void scan_kernel(
+__global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kernel(
     const T* __restrict__ in, T* __restrict__ out, int64_t n,
     int64_t in_stride, int64_t out_stride, int inclusive,
     uint32_t* __restrict__ ticket, TileState<T> st) {
@@ -299,7 +308,8 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
     const V* src = reinterpret_cast<const V*>(in + wave_base);
 #pragma unroll
     for (int j = 0; j < kTileVecs; ++j) {
-      V v = __builtin_nontemporal_load(&src[j * kWaveSize + lane]);
+      V v = ILGPU_HIP_SCAN_NT_LOAD ? __builtin_nontemporal_load(&src[j * kWaveSize + lane])
+                                   : src[j * kWaveSize + lane];
 #pragma unroll
       for (int k = 0; k < VN; ++k) x[j][k] = v[k];
     }
@@ -368,7 +378,8 @@ __global__ __launch_bounds__(kBlock, 4) void scan_kernel(
         V v;
 #pragma unroll
         for (int k = 0; k < VN; ++k) v[k] = r[k];
-        __builtin_nontemporal_store(v, &dst[j * kWaveSize + lane]);
+        if (ILGPU_HIP_SCAN_NT_STORE) __builtin_nontemporal_store(v, &dst[j * kWaveSize + lane]);
+        else dst[j * kWaveSize + lane] = v;
       } else {
 #pragma unroll
         for (int k = 0; k < VN; ++k) {
