@@ -176,8 +176,10 @@ static void section_copy() {
 
 // ------------------------------------------------------------- scatter ----
 // MODE 0: runs behind the previous tile's runs; 1: the same kernel writing its
-// tile linearly; C = 8, 16, 32: as 0, with chunks of C consecutive tiles kept
-// on one XCD (blocks are dealt to the eight XCDs round-robin).
+// tile linearly; 2: as 0, but every store instruction covers one 256-byte
+// aligned window of one run (lanes before the run's start are idle) and reads
+// what it stores from LDS; 10: as 2 with chunks of 8; C = 8, 16, 32: as 0, with chunks of C consecutive
+// tiles kept on one XCD (blocks are dealt to the eight XCDs round-robin).
 template <int BLOCK, int KPT, int MODE>
 __global__ __launch_bounds__(BLOCK) void scatter_runs(const uint32_t* __restrict__ src,
                                                       uint32_t* __restrict__ dst,
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(BLOCK) void scatter_runs(const uint32_t* __restrict
   uint32_t* s_start = s_len + 256;
   int t = blockIdx.x;
   if (MODE >= 8) {
-    constexpr int C = MODE;
+    constexpr int C = MODE == 10 ? 8 : MODE;
     const int xcd = blockIdx.x % 8, k = blockIdx.x / 8;
     const int tt = (8 * (k / C) + xcd) * C + k % C;
     if ((int)blockIdx.x < (int)(gridDim.x / (8 * C)) * 8 * C) t = tt;
@@ -227,6 +229,15 @@ __global__ __launch_bounds__(BLOCK) void scatter_runs(const uint32_t* __restrict
     for (uint32_t i = lane; i < n; i += 64) s_digit[p + i] = d;
   }
   __syncthreads();
+  if (MODE == 2 || MODE == 10) {
+    // every wave takes digits; its lanes sit on 256-byte windows of the destination
+    for (int d = wave; d < 256; d += BLOCK / 64) {
+      const uint32_t b = s_start[d], e = b + s_len[d];
+      for (uint32_t p = (b & ~63u) + lane; p < e; p += 64)
+        if (p >= b) dst[p] = key[0] + s_digit[p - s_off[d]];
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < KPT; ++j) {
     const int p = j * BLOCK + tid;
@@ -268,14 +279,18 @@ static void run_scatter(const char* name, int spread, const uint32_t* src, uint3
   const size_t lds = (size_t)(tile_keys + 4 * 256) * 4;
   CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 10>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   CK(hipFuncSetAttribute((const void*)scatter_runs<BLOCK, KPT, 32>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   const double bytes = 2.0 * (double)tiles * tile_keys * 4;
-  for (int mode : {1, 0, 8, 16, 32}) {
+  for (int mode : {1, 0, 2, 8, 10, 16, 32}) {
     const float ms = time_ms([&] {
       if (mode == 0) hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 0>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
       else if (mode == 1) hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 1>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
+      else if (mode == 2) hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 2>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
+      else if (mode == 10) hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 10>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
       else if (mode == 8) hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 8>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
       else if (mode == 16) hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 16>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
       else hipLaunchKernelGGL((scatter_runs<BLOCK, KPT, 32>), dim3(tiles), dim3(BLOCK), lds, 0, src, dst, dstart, dlen);
@@ -283,6 +298,8 @@ static void run_scatter(const char* name, int spread, const uint32_t* src, uint3
     char what[64];
     if (mode == 1) std::snprintf(what, sizeof what, "linear write");
     else if (mode == 0) std::snprintf(what, sizeof what, "256 runs per tile");
+    else if (mode == 2) std::snprintf(what, sizeof what, "256 runs per tile, aligned windows");
+    else if (mode == 10) std::snprintf(what, sizeof what, "256 runs, 8 per XCD, aligned windows");
     else std::snprintf(what, sizeof what, "256 runs, %d consecutive tiles per XCD", mode);
     std::printf("  %-38s %-40s %.3f ms  %.0f GB/s\n", name, what, ms, bytes / ms / 1e6);
   }

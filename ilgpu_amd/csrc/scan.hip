@@ -48,6 +48,16 @@ namespace {
 #ifndef ILGPU_HIP_SCAN_NT_STORE
 #define ILGPU_HIP_SCAN_NT_STORE 1
 #endif
+// Measurement only: 1 takes every tile's prefix as the identity (wrong results
+// beyond the first tile) to time the kernel without its look-back.
+#ifndef ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK
+#define ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK 0
+#endif
+// 1 issues the loads of a tile's second half only after the first half has
+// been scanned (half as many bytes in flight per wave).
+#ifndef ILGPU_HIP_SCAN_LOAD_HALVES
+#define ILGPU_HIP_SCAN_LOAD_HALVES 0
+#endif
 // 8-byte status words per tile: one 128-byte line each.  Every resident block
 // polls the words of the few dozen tiles before it with loads that go past the
 // L2; packed eight bytes apart those words share a handful of lines, and the
@@ -304,15 +314,19 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
                                        : kWaveElems);
 
   T x[kTileVecs][VN];
-  if (VECTOR && full) {
+  constexpr bool kHalves = ILGPU_HIP_SCAN_LOAD_HALVES && sizeof(T) == 4 && kTileVecs % 2 == 0;
+  auto load_rows = [&](int j0, int j1) {
     const V* src = reinterpret_cast<const V*>(in + wave_base);
 #pragma unroll
-    for (int j = 0; j < kTileVecs; ++j) {
+    for (int j = j0; j < j1; ++j) {
       V v = ILGPU_HIP_SCAN_NT_LOAD ? __builtin_nontemporal_load(&src[j * kWaveSize + lane])
                                    : src[j * kWaveSize + lane];
 #pragma unroll
       for (int k = 0; k < VN; ++k) x[j][k] = v[k];
     }
+  };
+  if (VECTOR && full) {
+    load_rows(0, kHalves ? kTileVecs / 2 : kTileVecs);
   } else {
 #pragma unroll
     for (int j = 0; j < kTileVecs; ++j)
@@ -357,7 +371,9 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
       block_total = F::apply(block_total, s_wave_total[w]);
     }
     if (wave == 0) {
-      const T exclusive = resolve_prefix<T, OP>(st, tile, block_total, lane);
+      const T exclusive = ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK
+                              ? F::identity()
+                              : resolve_prefix<T, OP>(st, tile, block_total, lane);
       if (lane == 0) s_prefix = exclusive;
     }
     __syncthreads();
@@ -394,13 +410,23 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
   // Lane-local inclusive scan of each vector, then one wave scan per j.
   T lane_excl[kTileVecs];   // fold of the vectors of lower lanes, same j
   T seg_total[kTileVecs];   // fold of the whole 64-lane row j
+  auto scan_rows = [&](int j0, int j1) {
 #pragma unroll
-  for (int j = 0; j < kTileVecs; ++j) {
+    for (int j = j0; j < j1; ++j) {
 #pragma unroll
-    for (int k = 1; k < VN; ++k) x[j][k] = F::apply(x[j][k - 1], x[j][k]);
-    const T inc = wave_inclusive_scan<T, OP>(x[j][VN - 1], lane);
-    seg_total[j] = shfl(inc, kWaveSize - 1);
-    lane_excl[j] = lane_shift_up<T>(F::identity(), inc);
+      for (int k = 1; k < VN; ++k) x[j][k] = F::apply(x[j][k - 1], x[j][k]);
+      const T inc = wave_inclusive_scan<T, OP>(x[j][VN - 1], lane);
+      seg_total[j] = shfl(inc, kWaveSize - 1);
+      lane_excl[j] = lane_shift_up<T>(F::identity(), inc);
+    }
+  };
+  if (kHalves && VECTOR && full) {
+    scan_rows(0, kTileVecs / 2);
+    __builtin_amdgcn_sched_barrier(0);
+    load_rows(kTileVecs / 2, kTileVecs);
+    scan_rows(kTileVecs / 2, kTileVecs);
+  } else {
+    scan_rows(0, kTileVecs);
   }
   T wave_total = seg_total[0];
 #pragma unroll
@@ -417,7 +443,9 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
   }
 
   if (wave == 0) {
-    const T exclusive = resolve_prefix<T, OP>(st, tile, block_total, lane);
+    const T exclusive = ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK
+                            ? F::identity()
+                            : resolve_prefix<T, OP>(st, tile, block_total, lane);
     if (lane == 0) s_prefix = exclusive;
   }
   __syncthreads();
@@ -437,7 +465,8 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
       V v;
 #pragma unroll
       for (int k = 0; k < VN; ++k) v[k] = r[k];
-      __builtin_nontemporal_store(v, &dst[j * kWaveSize + lane]);
+      if (ILGPU_HIP_SCAN_NT_STORE) __builtin_nontemporal_store(v, &dst[j * kWaveSize + lane]);
+      else dst[j * kWaveSize + lane] = v;
     } else {
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
