@@ -916,7 +916,7 @@ void onesweep_kernel(
   }
 }
 
-// ---- onesweep pass, pipelined form (integer keys only, large inputs) ----------
+// ---- onesweep pass, pipelined form (keys without values, large inputs) --------
 // The pass above runs a tile's phases one after the other: while a block waits
 // for its keys nothing else happens on its compute unit, and while it ranks,
 // walks and stages, no load is in flight.  This form overlaps them.
@@ -979,18 +979,22 @@ constexpr int kWalkDigits = kRadix / kWaveSize;       // digits per lane of a re
 
 // Loads the calling wave's keys of one tile into `key` and ranks them on the
 // wave's counters, which are zero on entry: as in sort_tile.
-template <int KEY_BYTES, bool FULL, bool HOT>
+template <int KEY_BYTES, bool FULL, bool HOT, bool FLOAT_KEYS>
 __device__ __forceinline__ void pipelined_rank(
     typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, 0))],
     uint32_t (&packed)[(items_per_thread(KEY_BYTES, 0)) / 2],
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int64_t tile_base, int valid,
-    int shift, typename KeyOf<KEY_BYTES>::type xor_mask, uint32_t* my_counters, int lane, int first_local,
+    int shift, const KeyXform& in_xf, uint32_t* my_counters, int lane, int first_local,
     const uint32_t (&hot)[kMaxHot]) {
   using K = typename KeyOf<KEY_BYTES>::type;
   constexpr int kItems = items_per_thread(KEY_BYTES, 0);
   load_tile_keys<KEY_BYTES, kItems, FULL>(src_keys, tile_base, valid, first_local, key);
+  // Float keys leave this function in their ordered form (in_xf is the
+  // identity when they arrive in it); integer keys keep their bits.
   auto item_digit = [&](int j) -> uint32_t {
-    const uint32_t d = (uint32_t)((K)(key[j] ^ xor_mask) >> shift) & (kRadix - 1);
+    if constexpr (FLOAT_KEYS) key[j] = ordered_bits(key[j], in_xf);
+    const K o = FLOAT_KEYS ? key[j] : (K)(key[j] ^ (K)in_xf.xor_mask);
+    const uint32_t d = (uint32_t)(o >> shift) & (kRadix - 1);
     return (FULL || first_local + j * kWaveSize < valid) ? d : (uint32_t)(kRadix - 1);
   };
   uint32_t hot_count[kMaxHot] = {};
@@ -1071,17 +1075,18 @@ __device__ __forceinline__ StatusVec load_status_row(__amdgpu_buffer_rsrc_t rsrc
                                                kStatusCoherent);
 }
 
-template <int KEY_BYTES>
+template <int KEY_BYTES, bool FLOAT_KEYS>
 __device__ __forceinline__ void pipelined_walk(
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int tile, int shift,
-    typename KeyOf<KEY_BYTES>::type xor_mask, __amdgpu_buffer_rsrc_t status,
+    const KeyXform& in_xf, __amdgpu_buffer_rsrc_t status,
     const uint32_t* __restrict__ excl_row, const uint32_t* s_total, const uint32_t* s_start,
     uint32_t* s_global_off, int lane, uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   constexpr int kTile = PipelinedTile<KEY_BYTES>::kTile;
   static_assert(kWalkDigits == 4, "a lane's digits are one 16-byte vector");
-  auto digit = [&](K k) -> uint32_t {
-    return (uint32_t)((K)(k ^ xor_mask) >> shift) & (kRadix - 1);
+  auto digit = [&](K k) -> uint32_t {  // of a key as the source holds it
+    const K o = FLOAT_KEYS ? ordered_bits(k, in_xf) : (K)(k ^ (K)in_xf.xor_mask);
+    return (uint32_t)(o >> shift) & (kRadix - 1);
   };
   const StatusVec my_count = reinterpret_cast<const StatusVec*>(s_total)[lane];
   const StatusVec my_excl = reinterpret_cast<const StatusVec*>(excl_row)[lane];
@@ -1184,10 +1189,10 @@ constexpr uint32_t kScannerPolls = 64;
 // prefixes written back.  A row's word either adds its count or (tile 0, or a
 // tile whose owner walked back itself) sets the running value.
 // s_lds: 16 + 17 x 64 words.
-template <int KEY_BYTES>
+template <int KEY_BYTES, bool FLOAT_KEYS>
 __device__ __forceinline__ void pipelined_scan(
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys, int shift,
-    typename KeyOf<KEY_BYTES>::type xor_mask, uint32_t* status, int num_tiles, uint32_t spin_limit,
+    const KeyXform& in_xf, uint32_t* status, int num_tiles, uint32_t spin_limit,
     uint32_t* s_lds) {
   using K = typename KeyOf<KEY_BYTES>::type;
   constexpr int kTile = PipelinedTile<KEY_BYTES>::kTile;
@@ -1305,8 +1310,9 @@ __device__ __forceinline__ void pipelined_scan(
       __syncthreads();
       const K* other = src_keys + (int64_t)t * kTile;
       for (int i = tid; i < kTile; i += kScanSegs * kWaveSize) {
-        K k = other[i];
-        atomicAdd(&s_part[(uint32_t)((K)(k ^ xor_mask) >> shift) & (kRadix - 1)], 1u);
+        const K k = other[i];
+        const K o = FLOAT_KEYS ? ordered_bits(k, in_xf) : (K)(k ^ (K)in_xf.xor_mask);
+        atomicAdd(&s_part[(uint32_t)(o >> shift) & (kRadix - 1)], 1u);
       }
       __syncthreads();
       if (seg == 0) s_prefix[lane] += s_part[dgt];
@@ -1319,7 +1325,7 @@ __device__ __forceinline__ void pipelined_scan(
   }
 }
 
-template <int KEY_BYTES>
+template <int KEY_BYTES, bool FLOAT_KEYS>
 __global__ __launch_bounds__(1024, ILGPU_HIP_SORT_WAVES_PER_EU)
 void onesweep_pipelined_kernel(
     typename KeyOf<KEY_BYTES>::type* keys_a, typename KeyOf<KEY_BYTES>::type* keys_b, int64_t n,
@@ -1354,11 +1360,20 @@ void onesweep_pipelined_kernel(
   const int shift = pass * 8;
   const uint32_t group = blockIdx.x % (uint32_t)groups;
   uint32_t* my_ticket = ticket + group * kTicketStride;
-  const K xor_mask = (K)xf.xor_mask;
+  // Float keys travel between the passes in their ordered form: the first pass
+  // that runs converts them as it ranks them, the last one converts them back
+  // as it writes them, and in between a digit is a shift and a mask (in_xf and
+  // out_xf are the identity then).  Integer keys keep their bits throughout;
+  // their order is one xor wherever a digit is taken.
+  KeyXform in_xf = xf, out_xf = xf;
+  if constexpr (FLOAT_KEYS) {
+    if (plan->first_executed != (uint32_t)pass) in_xf = KeyXform{0, 0, 0};
+    if (plan->last_executed != (uint32_t)pass) out_xf = KeyXform{0, 0, 0};
+  }
 
   if (with_scanner && blockIdx.x < kScanBlocks) {
     // ---- a scanning block: the prefixes of 64 digits ----
-    pipelined_scan<KEY_BYTES>(src_keys, shift, xor_mask, status, num_tiles,
+    pipelined_scan<KEY_BYTES, FLOAT_KEYS>(src_keys, shift, in_xf, status, num_tiles,
                                           spin_limit, s_counter);
     return;
   }
@@ -1418,7 +1433,7 @@ void onesweep_pipelined_kernel(
         }
       }
       if (!resolved)
-        pipelined_walk<KEY_BYTES>(src_keys, tile, shift, xor_mask, status_rows,
+        pipelined_walk<KEY_BYTES, FLOAT_KEYS>(src_keys, tile, shift, in_xf, status_rows,
                                               excl + pass * kRadix, s_total[par], s_start[par],
                                               s_global_off[par], lane, spin_limit);
       __syncthreads();  // this tile is resolved; the next one's totals are there, if there is one
@@ -1432,8 +1447,9 @@ void onesweep_pipelined_kernel(
   uint32_t hot[kMaxHot];
 #pragma unroll
   for (int h = 0; h < kMaxHot; ++h) hot[h] = plan->hot[pass][h];
-  auto digit = [&](K k) -> uint32_t {
-    return (uint32_t)((K)(k ^ xor_mask) >> shift) & (kRadix - 1);
+  auto digit = [&](K k) -> uint32_t {  // of a ranked or staged key
+    const K o = FLOAT_KEYS ? k : (K)(k ^ (K)xf.xor_mask);
+    return (uint32_t)(o >> shift) & (kRadix - 1);
   };
   auto arrive = [&](int which, int lane) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -1479,8 +1495,9 @@ void onesweep_pipelined_kernel(
       if (kFull || i < valid) {
         const K k = s_keys[i];
         const uint32_t g = global_off[digit(k)] + (uint32_t)i;
-        if (ILGPU_HIP_SORT_NT_STORE) __builtin_nontemporal_store(k, &dst_keys[g]);
-        else dst_keys[g] = k;
+        const K out = FLOAT_KEYS ? raw_bits(k, out_xf) : k;
+        if (ILGPU_HIP_SORT_NT_STORE) __builtin_nontemporal_store(out, &dst_keys[g]);
+        else dst_keys[g] = out;
       }
       if (j % ILGPU_HIP_SORT_WRITE_GROUP == ILGPU_HIP_SORT_WRITE_GROUP - 1)
         __builtin_amdgcn_sched_barrier(0);
@@ -1559,8 +1576,8 @@ void onesweep_pipelined_kernel(
       int tid = threadIdx.x;
       asm volatile("" : "+v"(tid));
       const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize;
-      pipelined_rank<KEY_BYTES, true, kHot>(
-          key, packed, src_keys, (int64_t)tile * kTile, kTile, shift, xor_mask, s_counter + wave * kRadix,
+      pipelined_rank<KEY_BYTES, true, kHot, FLOAT_KEYS>(
+          key, packed, src_keys, (int64_t)tile * kTile, kTile, shift, in_xf, s_counter + wave * kRadix,
           lane, wave * Cfg::kSubTileKeys + lane, hot);
     }
     bool ranked = true;
@@ -1571,8 +1588,8 @@ void onesweep_pipelined_kernel(
         int tid = threadIdx.x;
         asm volatile("" : "+v"(tid));
         const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize;
-        pipelined_rank<KEY_BYTES, true, kHot>(
-            key, packed, src_keys, (int64_t)next_tile * kTile, kTile, shift, xor_mask,
+        pipelined_rank<KEY_BYTES, true, kHot, FLOAT_KEYS>(
+            key, packed, src_keys, (int64_t)next_tile * kTile, kTile, shift, in_xf,
             s_counter + wave * kRadix, lane, wave * Cfg::kSubTileKeys + lane, hot);
       }
       tile = next_tile;
@@ -1590,8 +1607,8 @@ void onesweep_pipelined_kernel(
     last_valid = (int)(n - (int64_t)tile * kTile);
     K key[kItems];
     uint32_t packed[kItems / 2];
-    pipelined_rank<KEY_BYTES, false, true>(
-        key, packed, src_keys, (int64_t)tile * kTile, last_valid, shift, xor_mask,
+    pipelined_rank<KEY_BYTES, false, true, FLOAT_KEYS>(
+        key, packed, src_keys, (int64_t)tile * kTile, last_valid, shift, in_xf,
         s_counter + wave * kRadix, lane, wave * Cfg::kSubTileKeys + lane, hot);
     after_ranking(std::false_type{}, key, packed, last_valid);
   }
@@ -1900,7 +1917,11 @@ int32_t launch_passes_pipelined(hipStream_t stream, const SortArgs& a, const Tem
   uint32_t* excl = reinterpret_cast<uint32_t*>(base + L.excl);
   SortPlan* plan = reinterpret_cast<SortPlan*>(base + L.plan);
   uint32_t* tickets = reinterpret_cast<uint32_t*>(base + L.tickets);
-  auto* pass_kernel = onesweep_pipelined_kernel<KEY_BYTES>;
+  auto* pass_kernel = onesweep_pipelined_kernel<KEY_BYTES, false>;
+  if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
+    if ((xf.reference_term | xf.total_term) != 0)
+      pass_kernel = onesweep_pipelined_kernel<KEY_BYTES, true>;
+  }
   int64_t grid = cus;  // 1024 threads and 150 KiB of LDS: one block per compute unit
   if (grid > L.tiles) grid = L.tiles;
   const int groups = grid < kTicketGroups ? (int)grid : kTicketGroups;
@@ -1961,9 +1982,13 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
 #ifndef ILGPU_HIP_SORT_PIPELINED
 #define ILGPU_HIP_SORT_PIPELINED 1
 #endif
-  // Large keys-only sorts of integer keys take the pipelined form of the pass.
-  const bool use_pipelined = ILGPU_HIP_SORT_PIPELINED && VALUE_BYTES == 0 && use_large &&
-                             (xf.reference_term | xf.total_term) == 0;
+#ifndef ILGPU_HIP_SORT_PIPELINED_FLOAT
+#define ILGPU_HIP_SORT_PIPELINED_FLOAT 1
+#endif
+  // Large keys-only sorts take the pipelined form of the pass.
+  const bool use_pipelined =
+      ILGPU_HIP_SORT_PIPELINED && VALUE_BYTES == 0 && use_large &&
+      (ILGPU_HIP_SORT_PIPELINED_FLOAT || (xf.reference_term | xf.total_term) == 0);
   const TempLayout L =
       make_layout(a.n, KEY_BYTES, VALUE_BYTES, use_large ? kSortBlockLarge : kSortBlock,
                   use_pipelined ? pipelined_tile_keys(KEY_BYTES) : 0);

@@ -880,7 +880,7 @@ def test_sort_with_large_blocks_matches_oracle(large_sort_blocks, dtype, descend
 
 @pytest.mark.parametrize("dtype", [np.uint32, np.int32, np.uint64, np.int64, np.uint16, np.uint8])
 def test_sort_with_scanning_blocks_matches_numpy(large_sort_blocks, dtype):
-    # Integer keys in 1024-thread blocks take the pipelined form of the pass.
+    # Keys without values in 1024-thread blocks take the pipelined form of the pass.
     # From 64 tiles on, four blocks of the grid scan the tiles' digit counts
     # instead of sorting; below that every block resolves its tiles itself.
     # Sizes: some 100 tiles and a ragged last one; keys uniform, few-valued
@@ -901,6 +901,36 @@ def test_sort_with_scanning_blocks_matches_numpy(large_sort_blocks, dtype):
     assert np.array_equal(gpu_sort(const), const)
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+@pytest.mark.parametrize("descending", [False, True])
+def test_float_sort_with_scanning_blocks_matches_oracle(large_sort_blocks, dtype, descending):
+    # Float keys take the pipelined form too: the first pass that runs converts
+    # them to their ordered form as it ranks them, the last one converts them
+    # back as it writes them.  Arbitrary bit patterns (NaNs, infinities, both
+    # zeros), and inputs whose top or bottom passes are skipped, so that the
+    # converting passes are not the first and the last of the key.
+    items = 18 if np.dtype(dtype).itemsize == 8 else 36
+    tile = 15 * 64 * items
+    n = 66 * tile + 4321
+    rng = np.random.default_rng(11)
+    cases = [("bit patterns", random_float_bits(dtype, n, seed=5)),
+             ("one exponent", (1.0 + rng.random(n)).astype(dtype)),
+             ("coarse", (rng.integers(-8, 8, n) * 0.5).astype(dtype))]
+    for name, keys in cases:
+        note("pipelined float sort", np.dtype(dtype).name, descending, name, n)
+        assert bits_equal(gpu_sort(keys, descending=descending),
+                          O.radix_sort(keys, descending=descending)), name
+    u = {2: np.uint16, 4: np.uint32, 8: np.uint64}[np.dtype(dtype).itemsize]
+    keys = cases[0][1]
+    bits = keys.view(u)
+    sign = u(1) << u(np.dtype(dtype).itemsize * 8 - 1)
+    ordered = np.where(bits & sign, ~bits, bits | sign)
+    if descending:
+        ordered = ~ordered
+    expect = keys[np.argsort(ordered, kind="stable")]
+    assert bits_equal(gpu_sort(keys, descending=descending, float_total_order=True), expect)
+
+
 def test_sort_with_scanning_blocks_never_waits_without_bound(large_sort_blocks):
     # With the bound on polls at zero the scanning blocks count every tile they
     # find unpublished themselves, and the sorting blocks stop waiting for them
@@ -913,6 +943,12 @@ def test_sort_with_scanning_blocks_never_waits_without_bound(large_sort_blocks):
             note("pipelined sort, zero spin limit", np.dtype(dtype).name, n)
             keys = random_ints(dtype, n, seed=tiles)
             assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable")), n
+        # float keys: what a block counts itself comes from source keys that are
+        # raw in the first pass and ordered afterwards
+        n = 67 * 15 * 64 * 36 + 5
+        keys = random_float_bits(np.float32, n, seed=9)
+        note("pipelined float sort, zero spin limit", n)
+        assert bits_equal(gpu_sort(keys), O.radix_sort(keys))
     finally:
         capi.sort_set_parameter(capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT, -1)
 
