@@ -119,10 +119,17 @@ constexpr uint32_t kDefaultSpinLimit = 4096;
 // compute unit, which fill the GPU with fewer keys.
 constexpr int kSortBlock = ILGPU_HIP_SORT_BLOCK;      // small inputs, and the self-test
 constexpr int kSortBlockLarge = 1024;
-// The large block is used from this many of its tiles per compute unit on
-// (measured crossovers: 2^28 / 2^27 u32 keys gain 3 % / 1 %, 2^26 lose 4 %;
-// pairs of u64 keys and u32 values gain 4 to 8 % from 2^23 pairs on).
-constexpr int kLargeMinTilesPerCuKeys = 10;
+// The large block is used from this many of its tiles per compute unit on.
+// Keys without values take the pipelined pass there, measured against the
+// 512-thread classic pass on u32 keys (ms per sort): 2^24.6 keys (2.7 tiles
+// per CU) 0.291 / 0.277, 2^25 (3.6) 0.328 / 0.347, 2^25.6 (5.3) 0.461 / 0.480,
+// 2^26 (7.1) 0.572 / 0.617, 2^27 1.040 / 1.136.  The classic 1024-thread pass
+// (ILGPU_HIP_SORT_PIPELINED=0) pays from ten tiles per CU on; pairs of u64 keys
+// and u32 values gain 4 to 8 % from 2^23 pairs on.
+#ifndef ILGPU_HIP_SORT_PIPELINED
+#define ILGPU_HIP_SORT_PIPELINED 1
+#endif
+constexpr int kLargeMinTilesPerCuKeys = ILGPU_HIP_SORT_PIPELINED ? 3 : 10;
 constexpr int kLargeMinTilesPerCuPairs = 2;
 // Lanes that rank together (a sub-tile row): one wave.
 constexpr int kSubLanes = kWaveSize;
