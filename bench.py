@@ -248,7 +248,7 @@ def main():
                    "algorithmic_bytes_per_key": 4 * (2 * passes + 1)},
         "roofline": dict(roofline(pass_gbs, *measured_traffic(
                              "radix_sort_u32_uniform_2^28", args.log2n == 28)),
-                         kernel="onesweep_pipelined_kernel<4>",
+                         kernel="onesweep_pipelined_kernel<4, false>",
                          bytes_per_launch=pass_bytes,
                          avg_launch_ms=round(pass_ms, 4),
                          launches=pass_launches),
