@@ -1549,6 +1549,36 @@ def test_two_sorts_on_two_streams_share_the_gpu():
         assert np.array_equal(d_v[i].numpy(), order.astype(np.uint32)), i
 
 
+def test_two_pipelined_sorts_on_two_streams_share_the_gpu():
+    # Large keys-only sorts take the pipelined pass: one block per compute unit,
+    # four of them scanning.  Two such sorts on two streams cannot both be
+    # resident in full; a resolving wave polls its own row a bounded number of
+    # times and then walks back itself, and a scanning block counts a tile that
+    # nobody publishes, so both finish whatever the hardware interleaves.
+    import torch
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    n1, n2 = (1 << 25) + 11, (1 << 24) + 12345
+    a = datagen.uniform_u32(n1)
+    b = datagen.uniform_u64(n2)
+    d_a = [D.from_numpy(a) for _ in range(2)]
+    d_b = [D.from_numpy(b) for _ in range(2)]
+    t_a = [capi.temp_buffer(capi.radix_sort_temp_bytes(n1, np.uint32)) for _ in range(2)]
+    t_b = [capi.temp_buffer(capi.radix_sort_temp_bytes(n2, np.uint64)) for _ in range(2)]
+    torch.cuda.synchronize()
+    note("two pipelined sorts on two streams", n1, n2)
+    for i in range(2):
+        with torch.cuda.stream(s1):
+            capi.radix_sort_keys(d_a[i], t_a[i])
+        with torch.cuda.stream(s2):
+            capi.radix_sort_keys(d_b[i], t_b[i])
+    s1.synchronize()
+    s2.synchronize()
+    e_a, e_b = np.sort(a, kind="stable"), np.sort(b, kind="stable")
+    for i in range(2):
+        assert np.array_equal(d_a[i].numpy(), e_a), i
+        assert np.array_equal(d_b[i].numpy(), e_b), i
+
+
 def test_calls_can_be_captured_into_a_graph_and_replayed():
     # Every call is stream-ordered kernels only (temp memory is cleared by a
     # fill kernel, nothing is allocated), so a sequence of calls can be
