@@ -498,6 +498,9 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
 #ifndef ILGPU_HIP_UNIQUE_VECS
 #define ILGPU_HIP_UNIQUE_VECS 12
 #endif
+#ifndef ILGPU_HIP_UNIQUE_NT_STORE
+#define ILGPU_HIP_UNIQUE_NT_STORE 1
+#endif
 #ifndef ILGPU_HIP_UNIQUE_VECS1
 #define ILGPU_HIP_UNIQUE_VECS1 4
 #endif
@@ -619,7 +622,8 @@ __global__ __launch_bounds__(kBlock) void unique_kernel(
       V v;
 #pragma unroll
       for (int k = 0; k < VN; ++k) v[k] = x[j][k];
-      *reinterpret_cast<UnalignedV*>(data + pos) = v;
+      if (ILGPU_HIP_UNIQUE_NT_STORE) __builtin_nontemporal_store(v, reinterpret_cast<UnalignedV*>(data + pos));
+      else *reinterpret_cast<UnalignedV*>(data + pos) = v;
     } else {
 #pragma unroll
       for (int k = 0; k < VN; ++k)

@@ -93,17 +93,50 @@ __global__ __launch_bounds__(kBlock) void transform_kernel(
 // elements go through the scalar kernel.
 template <typename E, int K> struct alignas(sizeof(E) * K) Pack { E v[K]; };
 
+// Streaming (non-temporal) access to a pack as one machine vector of its size:
+// dense transforms read and write every byte once (negate of 2^28 int32:
+// 0.346 -> 0.33 ms).
+template <int BYTES> struct PackBits;
+template <> struct PackBits<2> { using type = uint16_t; };
+template <> struct PackBits<4> { using type = uint32_t; };
+template <> struct PackBits<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct PackBits<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+#ifndef ILGPU_HIP_TRANSFORM_NT
+#define ILGPU_HIP_TRANSFORM_NT 1
+#endif
+template <typename P> __device__ __forceinline__ P load_pack(const P* p) {
+  if constexpr (ILGPU_HIP_TRANSFORM_NT) {
+    using B = typename PackBits<sizeof(P)>::type;
+    const B bits = __builtin_nontemporal_load(reinterpret_cast<const B*>(p));
+    P out;
+    __builtin_memcpy(&out, &bits, sizeof(P));
+    return out;
+  } else {
+    return *p;
+  }
+}
+template <typename P> __device__ __forceinline__ void store_pack(P* p, const P& value) {
+  if constexpr (ILGPU_HIP_TRANSFORM_NT) {
+    using B = typename PackBits<sizeof(P)>::type;
+    B bits;
+    __builtin_memcpy(&bits, &value, sizeof(P));
+    __builtin_nontemporal_store(bits, reinterpret_cast<B*>(p));
+  } else {
+    *p = value;
+  }
+}
+
 template <typename S, typename T, int K>
 __global__ __launch_bounds__(kBlock) void transform_dense_kernel(
     const Pack<S, K>* source, Pack<T, K>* target, int64_t packs, int op, int64_t factor) {
   const int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < packs; i += step) {
-    const Pack<S, K> in = source[i];
+    const Pack<S, K> in = load_pack(&source[i]);
     Pack<T, K> out;
 #pragma unroll
     for (int k = 0; k < K; ++k)
       out.v[k] = convert<S, T>(apply_transformer<S>(in.v[k], op, factor));
-    target[i] = out;
+    store_pack(&target[i], out);
   }
 }
 
