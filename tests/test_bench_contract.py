@@ -60,3 +60,30 @@ def test_stale_counters_are_not_reported_as_traffic(tmp_path, monkeypatch):
     path.write_text(json.dumps(table))
     value, provenance = bench.measured_traffic("w", True)
     assert value == 5.0 and "stale" not in provenance
+
+
+def test_profile_summaries_name_commands_that_run_committed_files():
+    # Every summary under profiles/ gives the command that made it, and every
+    # file such a command runs is part of the repository (or is built from it
+    # by `python -m ilgpu_amd.build`: the library, its variants, bench_bounds).
+    import glob
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    summaries = sorted(glob.glob(os.path.join(root, "profiles", "*.txt")))
+    assert summaries
+    built = ("ilgpu_amd/lib/bench_bounds", "ilgpu_amd/lib/variants/")
+    for path in summaries:
+        text = open(path, encoding="utf-8").read()
+        assert "command" in text.split("\n\n")[0] + text, path
+        for name in re.findall(r"(?:python3?|--) +([\w/]+\.py)\b", text):
+            assert os.path.exists(os.path.join(root, name)), (path, name)
+        for name in re.findall(r"^\s+(ilgpu_amd/lib/[\w/]+)", text, flags=re.M):
+            assert name.startswith(built), (path, name)
+        assert "_work/" not in text, path
+
+
+def test_bounds_benchmark_is_part_of_the_build():
+    from ilgpu_amd import build
+    assert os.path.exists(build.BOUNDS_SRC)
+    if os.path.exists(build.LIB_PATH):
+        assert os.path.exists(build.BOUNDS_BIN), "python -m ilgpu_amd.build builds both"
