@@ -1659,8 +1659,13 @@ void onesweep_pipelined_kernel(
 // (lane l of wave w holds positions w*64*I + j*64 + l again), and the last pass
 // is followed by one coalesced write.  No histogram, plan, tickets, look-back
 // or temp memory; a pass whose digit is the same for every key simply leaves
-// the order as it is.
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS>
+// the order as it is.  ITEMS keys per thread: every row costs its rank, its
+// staging and its share of five barriers per pass whether it holds keys or
+// not, so short inputs take an instantiation with few rows (4, 12 or 24:
+// 32 to 2048 u32 keys 8 to 9 us instead of 24 to 27, up to 6144 keys 13
+// instead of 31).
+constexpr int kSmallSortItemsA = 4, kSmallSortItemsB = 12, kSmallSortItemsC = 24;
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, int ITEMS>
 __global__ __launch_bounds__(kSortBlock, ILGPU_HIP_SORT_WAVES_PER_EU)
 void small_sort_kernel(typename KeyOf<KEY_BYTES>::type* keys,
                        typename ValueOf<VALUE_BYTES>::type* vals, int n, KeyXform xf,
@@ -1668,13 +1673,18 @@ void small_sort_kernel(typename KeyOf<KEY_BYTES>::type* keys,
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
   using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, kSortBlock>;
-  constexpr int kItems = TileCfg::kItems;
+  constexpr int kItems = ITEMS;
   constexpr int kSubTiles = TileCfg::kSubTiles;
+  constexpr int kSubTileKeys = kSubLanes * kItems;
   constexpr bool kPairs = VALUE_BYTES > 0;
-  static_assert(!kPairs || TileCfg::kTile * VALUE_BYTES <= TileCfg::kStageBytes,
-                "the values of a tile are staged at once");
+  static_assert(kItems % 2 == 0 && kItems <= TileCfg::kItems, "ranks are packed in pairs");
+  // Counters, then the keys, then the values of the tile share these bytes.
+  constexpr int kEntryBytes = KEY_BYTES > VALUE_BYTES ? KEY_BYTES : VALUE_BYTES;
+  constexpr int kStageBytes = kSortBlock * kItems * kEntryBytes > TileCfg::kCounterBytes
+                                  ? kSortBlock * kItems * kEntryBytes
+                                  : TileCfg::kCounterBytes;
 
-  __shared__ __attribute__((aligned(16))) unsigned char s_stage[TileCfg::kStageBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[kStageBytes];
   __shared__ uint32_t s_scan[kRadix / kWaveSize];
   uint32_t* s_counter = reinterpret_cast<uint32_t*>(s_stage);
   K* s_keys = reinterpret_cast<K*>(s_stage);
@@ -1683,7 +1693,7 @@ void small_sort_kernel(typename KeyOf<KEY_BYTES>::type* keys,
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
   const int wave = tid / kWaveSize;
-  const int first_local = wave * TileCfg::kSubTileKeys + lane;
+  const int first_local = wave * kSubTileKeys + lane;
   uint32_t* my_counters = s_counter + wave * kRadix;
 
   K key[kItems];
@@ -1990,19 +2000,36 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
       g_sort_small_kernel.load(std::memory_order_relaxed) != 0) {
     // one tile: one block, one launch, no temp
     const KeyXform xf = make_xform(a.key_type, a.flags);
-    auto* kernel = small_sort_kernel<KEY_BYTES, VALUE_BYTES, false>;
-    if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
-      if ((xf.reference_term | xf.total_term) != 0)
-        kernel = small_sort_kernel<KEY_BYTES, VALUE_BYTES, true>;
+    constexpr int kFullItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
+    auto launch_small = [&](auto items) -> int32_t {
+      constexpr int kItems = decltype(items)::value;
+      auto* kernel = small_sort_kernel<KEY_BYTES, VALUE_BYTES, false, kItems>;
+      if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
+        if ((xf.reference_term | xf.total_term) != 0)
+          kernel = small_sort_kernel<KEY_BYTES, VALUE_BYTES, true, kItems>;
+      }
+      ProfileScope scope(stream, "sort_small");
+      hipLaunchKernelGGL(kernel, dim3(1), dim3(kSortBlock), 0, stream, static_cast<K*>(a.keys),
+                         static_cast<Val*>(a.values), (int)a.n, xf,
+                         a.value_source == ILGPU_HIP_VALUES_FROM_INDEX
+                               ? 1
+                               : (a.value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT ? 2 : 0));
+      ILGPU_HIP_CHECK(hipGetLastError());
+      return ILGPU_HIP_SUCCESS;
+    };
+    if constexpr (kSmallSortItemsA < kFullItems) {
+      if (a.n <= (int64_t)kSortBlock * kSmallSortItemsA)
+        return launch_small(std::integral_constant<int, kSmallSortItemsA>{});
     }
-    ProfileScope scope(stream, "sort_small");
-    hipLaunchKernelGGL(kernel, dim3(1), dim3(kSortBlock), 0, stream, static_cast<K*>(a.keys),
-                       static_cast<Val*>(a.values), (int)a.n, xf,
-                       a.value_source == ILGPU_HIP_VALUES_FROM_INDEX
-                             ? 1
-                             : (a.value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT ? 2 : 0));
-    ILGPU_HIP_CHECK(hipGetLastError());
-    return ILGPU_HIP_SUCCESS;
+    if constexpr (kSmallSortItemsB < kFullItems) {
+      if (a.n <= (int64_t)kSortBlock * kSmallSortItemsB)
+        return launch_small(std::integral_constant<int, kSmallSortItemsB>{});
+    }
+    if constexpr (kSmallSortItemsC < kFullItems) {
+      if (a.n <= (int64_t)kSortBlock * kSmallSortItemsC)
+        return launch_small(std::integral_constant<int, kSmallSortItemsC>{});
+    }
+    return launch_small(std::integral_constant<int, kFullItems>{});
   }
   const int cus = device_cu_count();
   int64_t min_tiles_per_cu = g_sort_large_min_tiles_per_cu.load(std::memory_order_relaxed);

@@ -878,6 +878,27 @@ def test_sort_with_large_blocks_matches_oracle(large_sort_blocks, dtype, descend
                           O.radix_sort(keys, descending=descending)), n
 
 
+@pytest.mark.parametrize("dtype", [np.uint32, np.int64, np.float32, np.float16, np.uint8])
+def test_one_tile_sort_at_the_edges_of_its_row_counts(dtype):
+    # Inputs of one tile are sorted by one block whose threads hold 4, 12, 24 or
+    # all of a tile's keys each, by the input's length: the lengths either side
+    # of every switch (512 threads x 4, 12, 24 keys; pairs switch where their
+    # shorter tiles allow).
+    for n in [2047, 2048, 2049, 6144, 6145, 12288, 12289]:
+        note("one-tile sort", np.dtype(dtype).name, n)
+        keys = (random_float_bits(dtype, n, seed=n) if np.dtype(dtype).kind == "f"
+                else random_ints(dtype, n, seed=n))
+        assert bits_equal(gpu_sort(keys), O.radix_sort(keys)), n
+        assert bits_equal(gpu_sort(keys, descending=True), O.radix_sort(keys, descending=True)), n
+    for n in [2048, 2049, 4095, 6144, 6145]:
+        # few distinct keys: stability decides the order of the values
+        keys = random_ints(np.int32, n, seed=n, lo=-9, hi=9).astype(dtype)
+        values = np.arange(n, dtype=np.uint32)
+        ek, ev = O.radix_sort_pairs(keys, values)
+        k, v = gpu_sort_pairs(keys, values)
+        assert bits_equal(k, ek) and np.array_equal(v, ev), n
+
+
 @pytest.mark.parametrize("dtype", [np.uint32, np.int32, np.uint64, np.int64, np.uint16, np.uint8])
 def test_sort_with_scanning_blocks_matches_numpy(large_sort_blocks, dtype):
     # Keys without values in 1024-thread blocks take the pipelined form of the pass.
