@@ -38,6 +38,7 @@ constexpr int kBlock = ILGPU_HIP_REDUCE_BLOCK;
 constexpr int kUnroll = ILGPU_HIP_REDUCE_UNROLL;
 constexpr int kMaxBlocks = 4096;  // upper bound on partials, fixes the temp size
 constexpr int kBlocksPerCu = ILGPU_HIP_REDUCE_BLOCKS_PER_CU;
+constexpr int64_t kSingleBlockElements = 32768;  // inputs up to here: one block, one launch
 
 template <typename T, int OP> struct AccType { using type = T; };
 template <> struct AccType<float, ILGPU_HIP_OP_ADD> { using type = double; };
@@ -60,7 +61,7 @@ __device__ __forceinline__ A block_fold(A v, A* lds) {
 template <typename T, int OP>
 __global__ __launch_bounds__(kBlock) void reduce_partials_kernel(
     const T* __restrict__ in, int64_t n, int64_t in_stride,
-    typename AccType<T, OP>::type* __restrict__ partials) {
+    typename AccType<T, OP>::type* __restrict__ partials, T* __restrict__ result) {
   using A = typename AccType<T, OP>::type;
   using F = Functor<A, OP>;
   using V = typename Vec16<T>::type;
@@ -75,7 +76,10 @@ __global__ __launch_bounds__(kBlock) void reduce_partials_kernel(
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step)
       acc = F::apply(acc, (A)in[i * in_stride]);
     A r = block_fold<A, OP>(acc, lds);
-    if (threadIdx.x == 0) partials[blockIdx.x] = r;
+    if (threadIdx.x == 0) {
+      if (result != nullptr) result[0] = (T)r;
+      else partials[blockIdx.x] = r;
+    }
     return;
   }
 
@@ -121,7 +125,11 @@ __global__ __launch_bounds__(kBlock) void reduce_partials_kernel(
 #pragma unroll
   for (int u = 1; u < kUnroll; ++u) acc[0] = F::apply(acc[0], acc[u]);
   A r = block_fold<A, OP>(acc[0], lds);
-  if (threadIdx.x == 0) partials[blockIdx.x] = r;
+  if (threadIdx.x == 0) {
+    // A launch of one block is the whole reduction: no second kernel.
+    if (result != nullptr) result[0] = (T)r;
+    else partials[blockIdx.x] = r;
+  }
 }
 
 template <typename T, int OP>
@@ -148,14 +156,19 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t n,
   if (blocks > cap) blocks = cap;
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
   if (blocks < 1) blocks = 1;
+  // Short inputs: one block folds everything and writes the result itself (a
+  // second launch costs more than the first block's extra elements).
+  if (n <= kSingleBlockElements) blocks = 1;
   A* partials = reinterpret_cast<A*>(align_up((int64_t)(uintptr_t)temp, 16));
   {
     ProfileScope scope(stream, "reduce_partials");
     hipLaunchKernelGGL((reduce_partials_kernel<T, OP>), dim3((unsigned)blocks),
                        dim3(kBlock), 0, stream, static_cast<const T*>(in), n,
-                       in_stride, partials);
+                       in_stride, partials,
+                       blocks == 1 ? static_cast<T*>(out) : static_cast<T*>(nullptr));
   }
   ILGPU_HIP_CHECK(hipGetLastError());
+  if (blocks == 1) return ILGPU_HIP_SUCCESS;
   {
     ProfileScope scope(stream, "reduce_final");
     hipLaunchKernelGGL((reduce_final_kernel<T, OP>), dim3(1), dim3(kBlock), 0,

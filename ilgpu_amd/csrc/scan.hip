@@ -298,9 +298,14 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
   __shared__ T s_wave_total[kWaves];
   __shared__ T s_prefix;
 
-  if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int tile = s_tile;
+  // An input of one tile comes without ticket and status words (and without
+  // the launch that clears them): there is nobody to wait for or to tell.
+  const bool alone = ticket == nullptr;
+  if (!alone) {
+    if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
+    __syncthreads();
+  }
+  const int tile = alone ? 0 : s_tile;
   const int lane = threadIdx.x & (kWaveSize - 1);
   // The wave index and everything derived from it are wave-uniform: kept in
   // scalar registers, so a lane addresses its vectors by one 32-bit offset.
@@ -371,7 +376,7 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
       block_total = F::apply(block_total, s_wave_total[w]);
     }
     if (wave == 0) {
-      const T exclusive = ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK
+      const T exclusive = ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK || alone
                               ? F::identity()
                               : resolve_prefix<T, OP>(st, tile, block_total, lane);
       if (lane == 0) s_prefix = exclusive;
@@ -443,7 +448,7 @@ __global__ __launch_bounds__(kBlock, ILGPU_HIP_SCAN_WAVES_PER_EU) void scan_kern
   }
 
   if (wave == 0) {
-    const T exclusive = ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK
+    const T exclusive = ILGPU_HIP_SCAN_PROBE_NO_LOOKBACK || alone
                             ? F::identity()
                             : resolve_prefix<T, OP>(st, tile, block_total, lane);
     if (lane == 0) s_prefix = exclusive;
@@ -541,9 +546,12 @@ __global__ __launch_bounds__(kBlock) void unique_kernel(
   __shared__ uint32_t s_wave_total[kWaves];
   __shared__ uint32_t s_prefix;
 
-  if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int tile = s_tile;
+  const bool alone = ticket == nullptr;  // one tile: no ticket, no status words
+  if (!alone) {
+    if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
+    __syncthreads();
+  }
+  const int tile = alone ? 0 : s_tile;
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int wave = threadIdx.x / kWaveSize;
   const int64_t tile_base = (int64_t)tile * kTile;
@@ -607,7 +615,7 @@ __global__ __launch_bounds__(kBlock) void unique_kernel(
   }
   if (wave == 0) {
     const uint32_t exclusive =
-        resolve_prefix<uint32_t, ILGPU_HIP_OP_ADD>(st, tile, block_total, lane);
+        alone ? 0u : resolve_prefix<uint32_t, ILGPU_HIP_OP_ADD>(st, tile, block_total, lane);
     if (lane == 0) s_prefix = exclusive;
   }
   __syncthreads();
@@ -655,10 +663,13 @@ int32_t launch_typed(hipStream_t stream, const void* in, int64_t in_stride,
   uint32_t* ticket = reinterpret_cast<uint32_t*>(base);
   TileState<T> st;
   st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
-  const int64_t zero_words = (kHeaderBytes + tiles * kStatusBytes) / 4;
-  int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
-                                 zero_words);
-  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  if (tiles > 1) {
+    const int64_t zero_words = (kHeaderBytes + tiles * kStatusBytes) / 4;
+    const int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base), zero_words);
+    if (rc != ILGPU_HIP_SUCCESS) return rc;
+  } else {
+    ticket = nullptr;  // one tile: one launch
+  }
   // Element strides above one (Stride1D.General) take the scalar path.
   const bool vector = in_stride == 1 && out_stride == 1 &&
                       (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
@@ -793,9 +804,13 @@ int32_t launch_unique_typed(hipStream_t stream, void* data, int64_t n,
   uint32_t* ticket = reinterpret_cast<uint32_t*>(base);
   TileState<uint32_t> st;
   st.words = reinterpret_cast<uint64_t*>(base + kHeaderBytes);
-  const int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
-                                       (kHeaderBytes + tiles * kStatusBytes) / 4);
-  if (rc != ILGPU_HIP_SUCCESS) return rc;
+  if (tiles > 1) {
+    const int32_t rc = launch_zero_words(stream, reinterpret_cast<uint32_t*>(base),
+                                         (kHeaderBytes + tiles * kStatusBytes) / 4);
+    if (rc != ILGPU_HIP_SUCCESS) return rc;
+  } else {
+    ticket = nullptr;  // one tile: one launch
+  }
   const bool vector = (reinterpret_cast<uintptr_t>(data) & 15) == 0;
   ProfileScope scope(stream, "unique");
   if (vector)
