@@ -974,7 +974,8 @@ void onesweep_kernel(
 //     which frees it): a wave clears its counters itself as soon as it has read
 //     its run starts, and no barrier separates positions from staging.
 //
-// Floating-point keys and pairs take the pass above.
+// Floating-point keys are converted by the first pass that runs and back by
+// the last one (in_xf, out_xf in the kernel); pairs take the pass above.
 template <int KEY_BYTES> struct PipelinedTile {
   static constexpr int kBlock = 1024;
   static constexpr int kSorterWaves = kBlock / kWaveSize - 1;
