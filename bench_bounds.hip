@@ -162,6 +162,13 @@ static void section_copy() {
   std::printf("  copy, one vector per thread, 256-thread blocks: %.4f ms  %.0f GB/s\n", ms, 2 * bytes / ms / 1e6);
   ms = time_ms([&] { hipLaunchKernelGGL((copy_stride<256, 4>), dim3(g_cus * 8), dim3(256), 0, 0, a, b, nvec); });
   std::printf("  copy, grid-stride, 256 threads x 4 vectors, 8 blocks per CU: %.4f ms  %.0f GB/s\n", ms, 2 * bytes / ms / 1e6);
+  run_copy_tile<256, 1, true>(a, b, nvec);
+  run_copy_tile<256, 2, true>(a, b, nvec);
+  run_copy_tile<256, 4, true>(a, b, nvec);
+  run_copy_tile<256, 8, true>(a, b, nvec);
+  run_copy_tile<1024, 1, true>(a, b, nvec);
+  run_copy_tile<1024, 2, true>(a, b, nvec);
+  run_copy_tile<1024, 4, true>(a, b, nvec);
   run_copy_tile<512, 16, true>(a, b, nvec);
   run_copy_tile<512, 16, false>(a, b, nvec);
   run_copy_tile<1024, 8, true>(a, b, nvec);
