@@ -73,8 +73,13 @@ def build(jobs: int | None = None) -> str:
 def build_variant(name: str, defines: list[str], units: list[str] | None = None) -> str:
     """Links a library whose `units` (file names in csrc/ without .hip; all of
     them when None) are compiled with -D<define> for every entry of `defines`;
-    the other units come from the objects of the last full build."""
+    the other units come from the objects of the last full build.  The units
+    that include radix_sort_impl.hpp go together: its macros size tiles, and the
+    temp size one unit reports has to be the layout another one writes."""
     all_sources = sources()
+    if units is not None and any(u.startswith("radix_sort") for u in units):
+        units = sorted(set(units) | {os.path.basename(s)[:-4] for s in all_sources
+                                     if os.path.basename(s).startswith("radix_sort")})
     chosen = [s for s in all_sources
               if units is None or os.path.basename(s)[:-4] in units]
     if units is not None and len(chosen) != len(units):
