@@ -349,6 +349,7 @@ SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0
 SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1
 SORT_PARAM_ONE_TILE_KERNEL = 2
 SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER = 3
+SORT_PARAM_SHORT_TILE_MAX_TILES = 4
 
 
 def sort_set_parameter(parameter: int, value: int) -> None:
@@ -356,6 +357,8 @@ def sort_set_parameter(parameter: int, value: int) -> None:
     LOOKBACK_SPIN_LIMIT: polls of an empty status word before a pass counts a
     missing tile itself (0 = at once: exercises the slow path).
     LARGE_BLOCK_MIN_TILES_PER_CU: 0 = always 1024-thread blocks, 2^31-1 = never.
+    SHORT_TILE_MAX_TILES: keys of at most this many full tiles take short tiles
+    (0 = never; at most the default, 512).
     ASSUME_LDS_ATOMIC_ORDER: 0 / 1 = every device counts as having failed / passed
     the check that precedes every sort; negative = ask the devices (anew)."""
     check(lib().ilgpu_hip_sort_set_parameter(parameter, value))

@@ -312,7 +312,8 @@ int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value) {
   if (parameter != ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT &&
       parameter != ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU &&
       parameter != ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL &&
-      parameter != ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER)
+      parameter != ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER &&
+      parameter != ILGPU_HIP_SORT_PARAM_SHORT_TILE_MAX_TILES)
     return ILGPU_HIP_ERROR_OUT_OF_RANGE;
   set_sort_parameter(parameter, value);
   return ILGPU_HIP_SUCCESS;

@@ -8,6 +8,7 @@ namespace ilgpu_hip {
 
 std::atomic<uint32_t> g_sort_spin_limit{kDefaultSpinLimit};
 std::atomic<int32_t> g_sort_large_min_tiles_per_cu{-1};
+std::atomic<int32_t> g_sort_short_tile_max_tiles{-1};
 std::atomic<int32_t> g_sort_small_kernel{1};
 // Test hook: -1 = ask the device (the default), 0 / 1 = every device is taken
 // to have failed / passed the check of its LDS atomics.
@@ -137,6 +138,8 @@ void set_sort_parameter(int32_t parameter, int32_t value) {
     g_sort_spin_limit.store(value < 0 ? kDefaultSpinLimit : (uint32_t)value, std::memory_order_relaxed);
   else if (parameter == ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU)
     g_sort_large_min_tiles_per_cu.store(value < 0 ? -1 : value, std::memory_order_relaxed);
+  else if (parameter == ILGPU_HIP_SORT_PARAM_SHORT_TILE_MAX_TILES)
+    g_sort_short_tile_max_tiles.store(value < 0 ? -1 : value, std::memory_order_relaxed);
   else
     g_sort_small_kernel.store(value == 0 ? 0 : 1, std::memory_order_relaxed);
 }

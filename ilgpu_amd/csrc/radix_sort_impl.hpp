@@ -55,6 +55,7 @@ namespace ilgpu_hip {
 extern std::atomic<uint32_t> g_sort_spin_limit;
 extern std::atomic<int32_t> g_sort_large_min_tiles_per_cu;  // negative: the defaults
 extern std::atomic<int32_t> g_sort_small_kernel;            // 0: one-tile inputs take the passes too
+extern std::atomic<int32_t> g_sort_short_tile_max_tiles;    // negative: the default
 
 namespace {
 
@@ -230,6 +231,23 @@ constexpr int items_per_thread(int key_bytes, int value_bytes) {
 }
 constexpr int tile_keys(int key_bytes, int value_bytes, int block) {
   return block * items_per_thread(key_bytes, value_bytes);
+}
+// Short tiles.  A sort of a few hundred tiles leaves compute units idle, and
+// each of its passes lasts as long as one tile takes from its first load to its
+// last store.  Keys without values that fit kShortTileMaxTiles tiles of a
+// shorter class (a third, a half or two thirds of the usual keys per thread)
+// take the shortest class that does: every tile resident at once, in one
+// round, more compute units at work and fewer rows to rank and to write per
+// block.
+#ifndef ILGPU_HIP_SORT_SHORT_TILE_MAX_TILES
+#define ILGPU_HIP_SORT_SHORT_TILE_MAX_TILES 512
+#endif
+constexpr int kShortTileMaxTiles = ILGPU_HIP_SORT_SHORT_TILE_MAX_TILES;
+constexpr int kShortTileClasses = 3;
+constexpr int short_items_per_thread(int key_bytes, int short_class) {
+  const int full = items_per_thread(key_bytes, 0);
+  const int items = short_class == 0 ? full / 3 : (short_class == 1 ? full / 2 : full * 2 / 3);
+  return items < 2 ? 2 : items & ~1;
 }
 
 // How raw key bits map to unsigned bits that sort in the requested order.
@@ -440,12 +458,14 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
 // checked on the device by ilgpu_hip_selftest_lds_atomic_order and, end to
 // end, by every stability test of the pair sorts.  With it the pass is stable
 // at one LDS operation per key and no cross-lane arithmetic.
-template <int KEY_BYTES, int VALUE_BYTES, int BLOCK> struct SortTile {
+template <int KEY_BYTES, int VALUE_BYTES, int BLOCK,
+          int ITEMS = items_per_thread(KEY_BYTES, VALUE_BYTES)>
+struct SortTile {
   static constexpr int kSubTiles = BLOCK / kSubLanes;
   static constexpr int kCounterWords = kSubTiles * kRadix;
   static constexpr int kCounterBytes = kCounterWords * 4;
-  static constexpr int kItems = items_per_thread(KEY_BYTES, VALUE_BYTES);
-  static constexpr int kTile = tile_keys(KEY_BYTES, VALUE_BYTES, BLOCK);
+  static constexpr int kItems = ITEMS;
+  static constexpr int kTile = BLOCK * ITEMS;
   static constexpr int kSubTileKeys = kSubLanes * kItems;
   static constexpr int kKeyStageBytes = kTile * KEY_BYTES;
   // The values of a tile go through the same LDS bytes after the keys, all at
@@ -513,9 +533,9 @@ __device__ __forceinline__ int ticket_tile(uint32_t k, uint32_t g, uint32_t grou
 }
 
 // Sorts one tile by the digit of `pass` and scatters it.
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT, int BLOCK>
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, bool FULL, bool HOT, int BLOCK, int ITEMS>
 __device__ __forceinline__ void sort_tile(
-    typename KeyOf<KEY_BYTES>::type (&key)[(items_per_thread(KEY_BYTES, VALUE_BYTES))],
+    typename KeyOf<KEY_BYTES>::type (&key)[ITEMS],
     const typename KeyOf<KEY_BYTES>::type* __restrict__ src_keys,
     typename KeyOf<KEY_BYTES>::type* __restrict__ dst_keys,
     const typename ValueOf<VALUE_BYTES>::type* __restrict__ src_vals,
@@ -526,7 +546,7 @@ __device__ __forceinline__ void sort_tile(
     const uint32_t (&hot)[kMaxHot], uint32_t spin_limit, bool in_raw, bool out_raw) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK, ITEMS>;
   constexpr int kItems = TileCfg::kItems;
   constexpr int kSubTiles = TileCfg::kSubTiles;
   constexpr bool kPairs = VALUE_BYTES > 0;
@@ -831,7 +851,7 @@ __device__ __forceinline__ void sort_tile(
   }
 }
 
-template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, int BLOCK>
+template <int KEY_BYTES, int VALUE_BYTES, bool FLOAT_KEYS, int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK, ILGPU_HIP_SORT_WAVES_PER_EU)
 void onesweep_kernel(
     typename KeyOf<KEY_BYTES>::type* keys_a,
@@ -843,7 +863,7 @@ void onesweep_kernel(
     int values_from_index, int groups, int chunk_shift, uint32_t spin_limit) {
   using K = typename KeyOf<KEY_BYTES>::type;
   using Val = typename ValueOf<VALUE_BYTES>::type;
-  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK>;
+  using TileCfg = SortTile<KEY_BYTES, VALUE_BYTES, BLOCK, ITEMS>;
   constexpr int kTile = TileCfg::kTile;
   constexpr int kItems = TileCfg::kItems;
 
@@ -888,13 +908,25 @@ void onesweep_kernel(
   // next keys during the look-back and the write-out, measured 3 to 12 % slower,
   // with the global ticket and again with the per-group ones.)  The key loads
   // fly while the ranking counters are cleared.
-  while (true) {
-    if (tid == 0) {
-      const uint32_t g = blockIdx.x % (uint32_t)groups;
-      s_tile = ticket_tile(atomicAdd(ticket + g * kTicketStride, 1u), g, (uint32_t)groups, chunk_shift);
+  // A grid of as many blocks as there are tiles (a short input) needs no
+  // tickets (ticket == nullptr): block b takes tile b and is done, which saves
+  // a pass two round trips to the ticket, one of them only to learn that
+  // there is nothing left.  Blocks are dispatched in index order, so a tile's
+  // predecessors have started; should they not be running, the bounded
+  // look-back covers that as it does with tickets.
+  for (int round = 0;; ++round) {
+    int tile;
+    if (ticket == nullptr) {
+      if (round > 0) break;
+      tile = (int)blockIdx.x;
+    } else {
+      if (tid == 0) {
+        const uint32_t g = blockIdx.x % (uint32_t)groups;
+        s_tile = ticket_tile(atomicAdd(ticket + g * kTicketStride, 1u), g, (uint32_t)groups, chunk_shift);
+      }
+      __syncthreads();  // also: the previous tile's staged keys have been read
+      tile = s_tile;
     }
-    __syncthreads();  // also: the previous tile's staged keys have been read
-    const int tile = s_tile;
     if (tile >= num_tiles) break;
     const int64_t tile_base = (int64_t)tile * kTile;
     const int valid = valid_keys(tile);
@@ -921,7 +953,7 @@ void onesweep_kernel(
           z[i] = make_uint4(0u, 0u, 0u, 0u);
       }
       __syncthreads();
-      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot, BLOCK>(
+      sort_tile<KEY_BYTES, VALUE_BYTES, FLOAT_KEYS, kFull, kHot, BLOCK, ITEMS>(
           key, src_keys, dst_keys, src_vals, dst_vals, tile_base, valid, tile, pass, xf, excl,
           status, make_index, s_stage, s_global_off, s_scan, hot, spin_limit, in_raw, out_raw);
     };
@@ -1842,10 +1874,30 @@ struct TempLayout {
 
 // Layout for tiles of `block` threads.  Temp views are sized for the small
 // block (more tiles, more status words); the large block's layout fits inside.
+// Keys per thread of the class of short tiles an input takes (the shortest
+// that makes at most `max_tiles` tiles), or 0: full tiles.
+inline int pick_short_items(int64_t n, int key_bytes, int value_bytes, int64_t max_tiles) {
+  if (value_bytes != 0) return 0;
+  // 8-byte keys: their full tiles are half as long to begin with, and beyond
+  // 128 short ones the longer look-back costs what the shorter tiles save.
+  if (key_bytes == 8 && max_tiles > kShortTileMaxTiles / 4) max_tiles = kShortTileMaxTiles / 4;
+  for (int c = 0; c < kShortTileClasses; ++c) {
+    const int items = short_items_per_thread(key_bytes, c);
+    if (div_up(n, (int64_t)kSortBlock * items) <= max_tiles) return items;
+  }
+  return 0;
+}
+// With the defaults (what temp views are sized by) the layout is that of the
+// shortest tiles the input can be given: the 512-thread block's, or short
+// tiles where they apply.
 TempLayout make_layout(int64_t n, int key_bytes, int value_bytes, int block = kSortBlock,
                        int64_t tile_override = 0) {
   TempLayout L;
-  const int64_t tile = tile_override > 0 ? tile_override : tile_keys(key_bytes, value_bytes, block);
+  int64_t tile = tile_override > 0 ? tile_override : tile_keys(key_bytes, value_bytes, block);
+  if (tile_override <= 0 && block == kSortBlock) {
+    const int short_items = pick_short_items(n, key_bytes, value_bytes, kShortTileMaxTiles);
+    if (short_items > 0) tile = (int64_t)kSortBlock * short_items;
+  }
   L.tiles = div_up(n, tile);
   int64_t off = 0;
   L.alt_keys = off; off += align_up(n * key_bytes, 256);
@@ -1889,8 +1941,9 @@ KeyXform make_xform(int32_t key_type, int32_t flags) {
   return xf;
 }
 
-// The passes of one sort with tiles of BLOCK threads.
-template <int KEY_BYTES, int VALUE_BYTES, int BLOCK>
+// The passes of one sort with tiles of BLOCK threads and ITEMS keys per thread.
+template <int KEY_BYTES, int VALUE_BYTES, int BLOCK,
+          int ITEMS = items_per_thread(KEY_BYTES, VALUE_BYTES)>
 int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L, char* base,
                       const KeyXform& xf, int cus) {
   using K = typename KeyOf<KEY_BYTES>::type;
@@ -1907,9 +1960,9 @@ int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L
                              ? 1
                              : (a.value_source == ILGPU_HIP_VALUES_FROM_INDEX_AS_FLOAT ? 2 : 0);
   const bool float_keys = (xf.reference_term | xf.total_term) != 0;
-  auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false, BLOCK>;
+  auto* pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, false, BLOCK, ITEMS>;
   if constexpr (KEY_BYTES >= 2) {  // there is no 1-byte floating-point key
-    if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true, BLOCK>;
+    if (float_keys) pass_kernel = onesweep_kernel<KEY_BYTES, VALUE_BYTES, true, BLOCK, ITEMS>;
   }
   // Resident blocks per CU of this instantiation: asked once per device and
   // kernel (the query costs microseconds, which small sorts would feel).
@@ -1943,8 +1996,9 @@ int32_t launch_passes(hipStream_t stream, const SortArgs& a, const TempLayout& L
       hipLaunchKernelGGL(pass_kernel,
                          dim3((unsigned)grid), dim3(BLOCK), 0, stream,
                          keys_a, keys_b, vals_a, vals_b, a.n, p, xf, excl,
-                         status, tickets + p * kTicketGroups * kTicketStride, plan, (int)L.tiles,
-                         from_index, groups, chunk_shift, spin_limit);
+                         status,
+                         grid == L.tiles ? nullptr : tickets + p * kTicketGroups * kTicketStride,
+                         plan, (int)L.tiles, from_index, groups, chunk_shift, spin_limit);
     }
     ILGPU_HIP_CHECK(hipGetLastError());
   }
@@ -2050,9 +2104,22 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   const bool use_pipelined =
       ILGPU_HIP_SORT_PIPELINED && VALUE_BYTES == 0 && use_large &&
       (ILGPU_HIP_SORT_PIPELINED_FLOAT || (xf.reference_term | xf.total_term) == 0);
+  // Short inputs of keys take short tiles (the parameter can only lower the
+  // limit: temp views are sized by the default).
+  int64_t short_max_tiles = g_sort_short_tile_max_tiles.load(std::memory_order_relaxed);
+  if (short_max_tiles < 0 || short_max_tiles > kShortTileMaxTiles)
+    short_max_tiles = kShortTileMaxTiles;
+  // Two 512-thread blocks are resident per compute unit; a second round of
+  // short tiles would cost more than full tiles do.
+  if (short_max_tiles > 2 * (int64_t)cus) short_max_tiles = 2 * (int64_t)cus;
+  const int short_items =
+      use_large ? 0 : pick_short_items(a.n, KEY_BYTES, VALUE_BYTES, short_max_tiles);
   const TempLayout L =
       make_layout(a.n, KEY_BYTES, VALUE_BYTES, use_large ? kSortBlockLarge : kSortBlock,
-                  use_pipelined ? pipelined_tile_keys(KEY_BYTES) : 0);
+                  use_pipelined ? pipelined_tile_keys(KEY_BYTES)
+                                : (short_items > 0 ? kSortBlock * short_items
+                                             : tile_keys(KEY_BYTES, VALUE_BYTES,
+                                                         use_large ? kSortBlockLarge : kSortBlock)));
   char* base = reinterpret_cast<char*>(align_up((int64_t)(uintptr_t)a.temp, 256));
   K* keys_a = static_cast<K*>(a.keys);
   K* keys_b = reinterpret_cast<K*>(base + L.alt_keys);
@@ -2075,7 +2142,14 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
            ((passes * kRadix) << (shift + 1)) <= kHistLdsWords)
       ++shift;
     const size_t lds = (size_t)((passes * kRadix) << shift) * 4;
-    int64_t blocks = div_up(div_up(a.n, Vec16<K>::N), kHistBlock);
+    // A block's fixed cost is its flush, one global atomic per digit value and
+    // position, which all blocks issue at about the same time.  Up to half a
+    // block per CU as soon as every thread has four vectors to count, more
+    // only when every thread has sixteen (2^20 u32 keys: 7.5 us instead of
+    // 15.5 with one vector per thread; 2^22: 12.3 instead of 17.1).
+    const int64_t vectors = div_up(a.n, Vec16<K>::N);
+    const int64_t few = std::min<int64_t>(div_up(vectors, kHistBlock * 4), std::max(cus / 2, 1));
+    int64_t blocks = std::max(few, div_up(vectors, kHistBlock * 16));
     // Two blocks of 64 KiB of counters are resident per CU: no second round.
     if (blocks > (int64_t)cus * ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU)
       blocks = (int64_t)cus * ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU;
@@ -2100,9 +2174,21 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
   if (use_pipelined) {
     if constexpr (VALUE_BYTES == 0)
       rc = launch_passes_pipelined<KEY_BYTES>(stream, a, L, base, xf, cus);
-  } else if (use_large)
+  } else if (use_large) {
     rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlockLarge>(stream, a, L, base, xf, cus);
-  else
+  } else if (short_items > 0) {
+    if constexpr (VALUE_BYTES == 0) {
+      constexpr int kA = short_items_per_thread(KEY_BYTES, 0);
+      constexpr int kB = short_items_per_thread(KEY_BYTES, 1);
+      constexpr int kC = short_items_per_thread(KEY_BYTES, 2);
+      if (short_items == kA)
+        rc = launch_passes<KEY_BYTES, 0, kSortBlock, kA>(stream, a, L, base, xf, cus);
+      else if (short_items == kB)
+        rc = launch_passes<KEY_BYTES, 0, kSortBlock, kB>(stream, a, L, base, xf, cus);
+      else
+        rc = launch_passes<KEY_BYTES, 0, kSortBlock, kC>(stream, a, L, base, xf, cus);
+    }
+  } else
     rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlock>(stream, a, L, base, xf, cus);
   if (rc != ILGPU_HIP_SUCCESS) return rc;
   {

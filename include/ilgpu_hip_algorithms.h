@@ -247,12 +247,19 @@ int32_t ilgpu_hip_sort_check_device(ilgpu_hip_stream_t stream);
  *   ASSUME_LDS_ATOMIC_ORDER  what ilgpu_hip_sort_check_device answers: 0 = every
  *     device is taken to have failed the check (sorts return
  *     ILGPU_HIP_ERROR_NOT_SUPPORTED before anything is launched), 1 = taken to
- *     have passed, negative (the default) = the devices are asked, anew. */
+ *     have passed, negative (the default) = the devices are asked, anew.
+ *   SHORT_TILE_MAX_TILES  keys without values are cut into 512-thread tiles of
+ *     a third, a half or two thirds of the usual length (6144, 9216 or 12288
+ *     keys of up to 4 bytes), the shortest that makes at most this many tiles:
+ *     more compute units at work on a short input.  Default 512, which is also
+ *     the most that is taken (temp sizes assume it), and never more than two
+ *     per compute unit; 0 = never. */
 enum {
   ILGPU_HIP_SORT_PARAM_LOOKBACK_SPIN_LIMIT = 0,
   ILGPU_HIP_SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU = 1,
   ILGPU_HIP_SORT_PARAM_ONE_TILE_KERNEL = 2,
-  ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER = 3
+  ILGPU_HIP_SORT_PARAM_ASSUME_LDS_ATOMIC_ORDER = 3,
+  ILGPU_HIP_SORT_PARAM_SHORT_TILE_MAX_TILES = 4
 };
 int32_t ilgpu_hip_sort_set_parameter(int32_t parameter, int32_t value);
 

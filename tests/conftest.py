@@ -40,5 +40,6 @@ def _sort_parameters_at_their_defaults():
         return
     for parameter in (capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT,
                       capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU,
-                      capi.SORT_PARAM_ONE_TILE_KERNEL):
+                      capi.SORT_PARAM_ONE_TILE_KERNEL,
+                      capi.SORT_PARAM_SHORT_TILE_MAX_TILES):
         capi.lib().ilgpu_hip_sort_set_parameter(parameter, -1)

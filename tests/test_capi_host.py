@@ -41,7 +41,7 @@ def test_temp_size_queries():
     keys_only = capi.radix_sort_temp_bytes(n, np.uint32)
     assert keys_only >= n * 4
     with_values = capi.radix_sort_temp_bytes(n, np.uint32, 4)
-    assert with_values >= keys_only + n * 4
+    assert with_values >= n * 8  # alternate buffers for keys and values
     # 2^27 pairs of (u64, u32): the size the reference's own helper overflows
     # on (RadixSortExtensions.cs:400-402) is computed in 64 bits here.
     big = capi.radix_sort_temp_bytes(1 << 27, np.uint64, 4)

@@ -774,6 +774,11 @@ def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
         k, v = gpu_sort_pairs(keys, values)
         order = np.argsort(keys, kind="stable")
         assert np.array_equal(k, keys[order]) and np.array_equal(v, values[order])
+        # the same with full tiles where short ones are the default
+        capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, 0)
+        keys = random_ints(np.uint32, 18432 * 40 + 77, seed=19)
+        assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+        capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, -1)
         # the same with 1024-thread blocks
         capi.sort_set_parameter(capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU, 0)
         keys = random_ints(np.uint32, 36864 * 20 + 77, seed=17)
@@ -786,6 +791,7 @@ def test_sort_look_back_that_never_waits_counts_missing_tiles_itself():
     finally:
         capi.sort_set_parameter(capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT, -1)
         capi.sort_set_parameter(capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU, -1)
+        capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, -1)
     # back on the defaults
     keys = random_ints(np.uint32, 18432 * 40 + 77, seed=16)
     assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
@@ -876,6 +882,68 @@ def test_sort_with_large_blocks_matches_oracle(large_sort_blocks, dtype, descend
         keys = random_float_bits(dtype, n, seed=n) if kinds == "f" else random_ints(dtype, n, seed=n)
         assert bits_equal(gpu_sort(keys, descending=descending),
                           O.radix_sort(keys, descending=descending)), n
+
+
+# Keys without values that make at most 512 tiles (128 with 8-byte keys) of a
+# shorter class (512 threads x 12, 18 or 24 keys of up to 4 bytes; 6, 8 or 12 of
+# 8 bytes) take the shortest class that does, every block one tile without a
+# ticket; longer inputs and pairs take full tiles.
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_with_short_tiles_matches_oracle(dtype, descending):
+    kinds = np.dtype(dtype).kind
+    for n in [18433, 30000, 6144 * 7 + 5, 3072 * 9 - 1, 100003, 400001]:
+        note("short-tile sort", np.dtype(dtype).name, descending, n)
+        keys = random_float_bits(dtype, n, seed=n) if kinds == "f" else random_ints(dtype, n, seed=n)
+        assert bits_equal(gpu_sort(keys, descending=descending),
+                          O.radix_sort(keys, descending=descending)), n
+
+
+@pytest.mark.parametrize("dtype,sizes", [
+    (np.uint32, [512 * 6144, 512 * 6144 + 1, 512 * 9216, 512 * 9216 + 1, 512 * 12288,
+                 512 * 12288 + 1]),
+    (np.int16, [512 * 6144 - 1, 512 * 9216 + 1, 512 * 12288 + 1]),
+    (np.uint64, [128 * 3072, 128 * 3072 + 1, 128 * 4096, 128 * 4096 + 1, 128 * 6144,
+                 128 * 6144 + 1])])
+def test_sort_at_the_edges_of_the_short_tile_classes(dtype, sizes):
+    # the longest input of every class and the shortest of the next one
+    for n in sizes:
+        note("short-tile class edge", np.dtype(dtype).name, n)
+        keys = random_ints(dtype, n, seed=n & 0xFFFF)
+        assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable")), n
+
+
+@pytest.fixture
+def no_short_tiles():
+    """Short inputs of keys take full tiles like pairs and longer inputs do."""
+    capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, 0)
+    yield
+    capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, -1)
+
+
+@pytest.mark.parametrize("dtype", ALL_KEY_DTYPES)
+def test_sort_of_short_inputs_with_full_tiles_matches_oracle(no_short_tiles, dtype):
+    kinds = np.dtype(dtype).kind
+    for n in [18433, 100003, 18432 * 12 + 77]:
+        note("short input, full tiles", np.dtype(dtype).name, n)
+        keys = random_float_bits(dtype, n, seed=n) if kinds == "f" else random_ints(dtype, n, seed=n)
+        for descending in (False, True):
+            assert bits_equal(gpu_sort(keys, descending=descending),
+                              O.radix_sort(keys, descending=descending)), (n, descending)
+
+
+def test_sort_with_more_tiles_than_blocks_draws_tickets():
+    # 515 full tiles of keys and 600 of pairs on at most 512 resident blocks:
+    # the blocks draw their tiles from the tickets, some of them two.
+    n = 18432 * 515 + 3
+    keys = random_ints(np.uint32, n, seed=21)
+    assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+    n = 8192 * 600 + 3
+    keys = random_ints(np.uint32, n, seed=22, lo=0, hi=4999)
+    values = np.arange(n, dtype=np.uint32)
+    k, v = gpu_sort_pairs(keys, values)
+    order = np.argsort(keys, kind="stable")
+    assert np.array_equal(k, keys[order]) and np.array_equal(v, values[order])
 
 
 @pytest.mark.parametrize("dtype", [np.uint32, np.int64, np.float32, np.float16, np.uint8])
