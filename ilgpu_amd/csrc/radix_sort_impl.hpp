@@ -393,11 +393,18 @@ __global__ __launch_bounds__(kRadix) void plan_kernel(
   const int lane = d & (kWaveSize - 1);
   const int wave = d / kWaveSize;
   uint32_t parity = 0, executed = 0, first = passes, last = passes;
-  for (int p = 0; p < passes; ++p) {
+  // The counts of every pass in one round trip (the loop below is a chain of
+  // barriers that a load inside it would wait behind, pass after pass).
+  uint32_t counts[kMaxPasses];
+#pragma unroll
+  for (int p = 0; p < kMaxPasses; ++p) counts[p] = p < passes ? global_hist[p * kRadix + d] : 0u;
+#pragma unroll
+  for (int p = 0; p < kMaxPasses; ++p) {
+    if (p >= passes) break;
     if (d < kMaxHot) s_hot[d] = 0ull;
     if (d == 0) s_trivial = 0;
     __syncthreads();
-    const uint32_t c = global_hist[p * kRadix + d];
+    const uint32_t c = counts[p];
     if (c == n) s_trivial = 1;
     // A digit qualifies with an eighth of the keys (two lanes of a
     // sub-tile row on average); kMaxHot rounds of "largest below the previous
