@@ -2199,7 +2199,9 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
     rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlock>(stream, a, L, base, xf, cus);
   if (rc != ILGPU_HIP_SUCCESS) return rc;
   {
-    int64_t blocks = div_up(a.n, 256);
+    // Mostly there is nothing to copy and every block returns at once: a
+    // short input gets a grid that is dispatched quickly (16 keys per thread).
+    int64_t blocks = div_up(a.n, 256 * 16);
     if (blocks > (int64_t)cus * 8) blocks = (int64_t)cus * 8;
     ProfileScope scope(stream, "sort_finish");
     hipLaunchKernelGGL((finish_kernel<KEY_BYTES, VALUE_BYTES>),
