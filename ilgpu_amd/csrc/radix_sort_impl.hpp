@@ -141,6 +141,9 @@ constexpr int kLookback = ILGPU_HIP_SORT_LOOKBACK;
 #ifndef ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU
 #define ILGPU_HIP_SORT_HIST_BLOCKS_PER_CU 2
 #endif
+#ifndef ILGPU_HIP_SORT_HIST_RUNS
+#define ILGPU_HIP_SORT_HIST_RUNS 1
+#endif
 #ifndef ILGPU_HIP_SORT_HIST_NT
 #define ILGPU_HIP_SORT_HIST_NT 1
 #endif
@@ -305,6 +308,22 @@ struct SortPlan {
   uint32_t final_in_alt;            // result sits in the alternate buffer
 };
 
+// The first active lane's key, as a wave-uniform value.
+__device__ __forceinline__ uint64_t readfirstlane_key(uint64_t k) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)k);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(k >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint32_t readfirstlane_key(uint32_t k) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)k);
+}
+__device__ __forceinline__ uint32_t readfirstlane_key(uint16_t k) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)k);
+}
+__device__ __forceinline__ uint32_t readfirstlane_key(uint8_t k) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)k);
+}
+
 // ---- histogram of all digit positions ------------------------------------
 template <typename K, bool FLOAT_KEYS>
 __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
@@ -339,6 +358,76 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
   auto load_keys = [](const V* p) -> V {
     return ILGPU_HIP_SORT_HIST_NT ? __builtin_nontemporal_load(p) : *p;
   };
+  // Vectors whose keys are the same in every lane of a wave, wholly or in their
+  // upper half (constant input; small values under large types), would meet
+  // in one counter 256 keys deep.  They are counted as runs in registers, one
+  // check per vector, and reach the counters when the value changes; only
+  // with all 64 lanes at work, so that the run is the same in every lane.
+  // (Sorts of 2^28 u32 keys: all equal 0.269 -> 0.197 ms, Zipf values below
+  // 2^16 1.174 -> 1.120, uniform 2.056 -> 2.059.)
+  constexpr int kHalfBits = 4 * (int)sizeof(K);
+  K run_key = 0, run_half = 0;
+  uint32_t run_key_count = 0, run_half_count = 0;
+  auto flush_key_run = [&]() {
+    if ((threadIdx.x & (kWaveSize - 1)) == 0 && run_key_count != 0u) {
+      K o = (K)(run_key ^ (K)xf.xor_mask);
+      if constexpr (FLOAT_KEYS) o ^= key_term(run_key, xf);
+#pragma unroll
+      for (int p = 0; p < (int)sizeof(K); ++p)
+        atomicAdd(&s_hist[((p * kRadix + ((uint32_t)(o >> (8 * p)) & (kRadix - 1))) << replica_shift) + replica],
+                  run_key_count);
+    }
+    run_key_count = 0u;
+  };
+  auto flush_half_run = [&]() {  // run_half: ordered bits above the lower half
+    if ((threadIdx.x & (kWaveSize - 1)) == 0 && run_half_count != 0u) {
+#pragma unroll
+      for (int p = (int)sizeof(K) / 2; p < (int)sizeof(K); ++p)
+        atomicAdd(&s_hist[((p * kRadix + ((uint32_t)(run_half >> (8 * p - kHalfBits)) & (kRadix - 1))) << replica_shift) + replica],
+                  run_half_count);
+    }
+    run_half_count = 0u;
+  };
+  // Whether a vector's keys agree in every lane of the (full) wave: wholly
+  // (returns 2), in their upper half (1), or not (0).
+  auto uniformity = [&](const V& v, K& first) -> int {
+    K diff = 0;
+#pragma unroll
+    for (int k = 1; k < VN; ++k) diff |= (K)(v[k] ^ v[0]);
+    first = (K)readfirstlane_key(v[0]);
+    diff |= (K)(v[0] ^ first);
+    if (__ballot(true) != ~0ull) return 0;
+    if (__ballot(diff != 0) == 0ull) return 2;
+    if (FLOAT_KEYS) return 0;  // the upper half of their ordered bits depends on the sign
+    return __ballot((K)(diff >> kHalfBits) != 0) == 0ull ? 1 : 0;
+  };
+  auto count_vector = [&](auto checked, const V& v) {
+    if constexpr (decltype(checked)::value) {
+      K first;
+      const int same = uniformity(v, first);
+      if (same == 2) {
+        if (first != run_key) { flush_key_run(); run_key = first; }
+        run_key_count += (uint32_t)(kWaveSize * VN);
+        return;
+      }
+      if (same == 1) {
+        const K half = (K)((K)(first ^ (K)xf.xor_mask) >> kHalfBits);
+        if (half != run_half) { flush_half_run(); run_half = half; }
+        run_half_count += (uint32_t)(kWaveSize * VN);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          const K o = (K)(v[k] ^ (K)xf.xor_mask);
+#pragma unroll
+          for (int p = 0; p < (int)sizeof(K) / 2; ++p)
+            atomicAdd(&s_hist[((p * kRadix + ((uint32_t)(o >> (8 * p)) & (kRadix - 1))) << replica_shift) + replica], 1u);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < VN; ++k) count(v[k]);
+  };
   const uintptr_t addr = reinterpret_cast<uintptr_t>(keys);
   int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(K));
   if (head > n) head = n;
@@ -346,22 +435,41 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
   const int64_t nvec = (n - head) / VN;
   const int64_t tail_start = head + nvec * VN;
   const int64_t stride = (int64_t)gridDim.x * kHistBlock;
+  // The first round's vectors are requested, and by the first of them a wave
+  // decides whether it looks for runs at all: the check costs keys that vary
+  // 1 to 2 % of a sort when every vector pays it.
   int64_t i = (int64_t)blockIdx.x * kHistBlock + threadIdx.x;
-  for (; i + (kHistUnroll - 1) * stride < nvec; i += kHistUnroll * stride) {
-    V v[kHistUnroll];
+  V v0[kHistUnroll];
+  const bool have_first = i + (kHistUnroll - 1) * stride < nvec;
+  if (have_first) {
 #pragma unroll
-    for (int u = 0; u < kHistUnroll; ++u) v[u] = load_keys(&body[i + u * stride]);
+    for (int u = 0; u < kHistUnroll; ++u) v0[u] = load_keys(&body[i + u * stride]);
+  }
+  bool look_for_runs = false;
+  if (ILGPU_HIP_SORT_HIST_RUNS && sizeof(K) >= 2 && have_first) {
+    K first;
+    look_for_runs = uniformity(v0[0], first) != 0;
+  }
+  auto count_body = [&](auto checked) {
+    if (have_first) {
 #pragma unroll
-    for (int u = 0; u < kHistUnroll; ++u) {
-#pragma unroll
-      for (int k = 0; k < VN; ++k) count(v[u][k]);
+      for (int u = 0; u < kHistUnroll; ++u) count_vector(checked, v0[u]);
+      i += kHistUnroll * stride;
     }
-  }
-  for (; i < nvec; i += stride) {
-    V a = load_keys(&body[i]);
+    for (; i + (kHistUnroll - 1) * stride < nvec; i += kHistUnroll * stride) {
+      V v[kHistUnroll];
 #pragma unroll
-    for (int k = 0; k < VN; ++k) count(a[k]);
-  }
+      for (int u = 0; u < kHistUnroll; ++u) v[u] = load_keys(&body[i + u * stride]);
+#pragma unroll
+      for (int u = 0; u < kHistUnroll; ++u) count_vector(checked, v[u]);
+    }
+    for (; i < nvec; i += stride) {
+      V a = load_keys(&body[i]);
+      count_vector(checked, a);
+    }
+  };
+  if (look_for_runs) count_body(std::true_type{});
+  else count_body(std::false_type{});
   if (blockIdx.x == 0) {
     const int64_t extra = head + (n - tail_start);
     if ((int64_t)threadIdx.x < extra) {
@@ -371,6 +479,8 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
       count(keys[idx]);
     }
   }
+  flush_key_run();
+  flush_half_run();
   __syncthreads();
 
   const int replicas = 1 << replica_shift;

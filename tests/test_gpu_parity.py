@@ -913,6 +913,57 @@ def test_sort_at_the_edges_of_the_short_tile_classes(dtype, sizes):
         assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable")), n
 
 
+@pytest.mark.parametrize("dtype", [np.uint16, np.uint32, np.int32, np.uint64, np.int64,
+                                   np.float32, np.float64])
+def test_sort_of_keys_that_agree_across_whole_waves(dtype):
+    # The digit histogram counts vectors whose keys agree in every lane of a wave
+    # (wholly, or in their upper half) as runs in registers; a wave looks for
+    # them when its first vector is one.  Stretches of constant keys, of small
+    # values and of varying keys, with odd lengths so that the stretches start
+    # and end inside vectors and waves, in either order, and a view that starts
+    # off a 16-byte boundary.
+    dt = np.dtype(dtype)
+    rng = np.random.default_rng(77)
+    bits = dt.itemsize * 8
+    udt = np.dtype(f"u{dt.itemsize}")
+
+    def varying(m):
+        return rng.integers(0, 1 << bits, size=m, dtype=np.uint64).astype(udt)
+
+    def small(m):
+        return rng.integers(0, 1 << (bits // 2), size=m, dtype=np.uint64).astype(udt)
+
+    def constant(m, value):
+        return np.full(m, value & ((1 << bits) - 1), dtype=udt)
+
+    for order in (0, 1):
+        parts = [constant(70001, 0xDEADBEEFCAFEF00D), constant(30011, 5), small(130003),
+                 varying(90007), constant(50021, 0x8000000000000001), small(40009)]
+        if order:
+            parts = [varying(4099)] + parts[::-1]
+        raw = np.concatenate(parts)
+        if dt.kind == "f":   # no NaN payload games here: keep every exponent finite
+            raw &= udt.type(~(1 << (bits - 2)) & ((1 << bits) - 1))
+        keys = raw.view(dt)
+        for off in (0, 1):
+            k = keys[off:]
+            note("keys that agree across waves", dt.name, order, off, k.size)
+            big = D.from_numpy(keys)
+            view = D(k.size, dt, _bytes=big.bytes[off * dt.itemsize:])
+            capi.radix_sort_keys(view)
+            sync()
+            got = view.numpy()
+            if dt.kind == "f":
+                assert bits_equal(got, O.radix_sort(k)), (order, off)
+            else:
+                assert np.array_equal(got, np.sort(k, kind="stable")), (order, off)
+    # long enough for the grid to have every block several rounds deep
+    n = (1 << 23) + 12345
+    keys = np.concatenate([constant(n // 2, 0x1234567812345678), small(n - n // 2)]).view(dt)
+    if dt.kind != "f":
+        assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
+
+
 @pytest.fixture
 def no_short_tiles():
     """Short inputs of keys take full tiles like pairs and longer inputs do."""
