@@ -18,7 +18,11 @@
 //            wave, on an idle device and on a compute unit that is streaming
 //            keys: what a look-back step costs.
 //
-// Usage: bench_bounds [copy|scatter|lds|latency|all]   (default all)
+//   tiles    blocks per microsecond with and without a ticket, and a tile-shaped
+//            read of 1 GiB behind it: what scan and unique pay per tile before
+//            any arithmetic.
+//
+// Usage: bench_bounds [copy|scatter|lds|latency|tiles|all]   (default all)
 // Built by `python -m ilgpu_amd.build` into ilgpu_amd/lib/bench_bounds.
 #include <hip/hip_runtime.h>
 
@@ -574,6 +578,72 @@ static void section_latency() {
   CK(hipFree(b));
 }
 
+// --------------------------------------------------------------- tiles ----
+// What a single-pass kernel pays per tile before any arithmetic: the dispatch
+// of a 512-thread block, the ticket that orders the tiles (one returning atomic
+// on one address, which the whole block waits for) and the tile's loads.
+template <bool TICKET, int VECS>
+__global__ __launch_bounds__(512) void tile_read(const u32x4* __restrict__ in, uint32_t* ticket,
+                                                 uint32_t* sink) {
+  __shared__ uint32_t s_tile;
+  uint32_t tile = blockIdx.x;
+  if (TICKET) {
+    if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
+    __syncthreads();
+    tile = s_tile;
+  }
+  if (VECS == 0) return;
+  const u32x4* base = in + (size_t)tile * (512 * (VECS > 0 ? VECS : 1));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  u32x4 v[VECS > 0 ? VECS : 1];
+#pragma unroll
+  for (int j = 0; j < VECS; ++j)
+    v[j] = __builtin_nontemporal_load(&base[(wave * VECS + j) * 64 + lane]);
+  uint32_t x = 0;
+#pragma unroll
+  for (int j = 0; j < VECS; ++j) x ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+  if (x == 0x9E3779B9u) sink[0] = x;  // never true for the data used: keeps the loads
+}
+
+template <bool TICKET, int VECS>
+static void run_tile_read(const u32x4* in, uint32_t* ticket, uint32_t* sink, int tiles) {
+  const float ms = time_ms([&] {
+    if (TICKET) CK(hipMemsetAsync(ticket, 0, 4));
+    hipLaunchKernelGGL((tile_read<TICKET, VECS>), dim3(tiles), dim3(512), 0, 0, in, ticket, sink);
+  });
+  if (VECS == 0)
+    std::printf("  %6d blocks, %-9s no loads                : %.4f ms  %5.1f blocks per us\n", tiles,
+                TICKET ? "ticket," : "no ticket,", ms, tiles / ms / 1e3);
+  else
+    std::printf("  %6d blocks, %-9s %2d vectors per thread    : %.4f ms  %5.1f blocks per us  %5.0f GB/s\n",
+                tiles, TICKET ? "ticket," : "no ticket,", VECS, ms, tiles / ms / 1e3,
+                (double)tiles * 512 * VECS * 16 / ms / 1e6);
+}
+
+static void section_tiles() {
+  const size_t nvec = (size_t)1 << 26;  // 1 GiB
+  u32x4* in;
+  uint32_t *ticket, *sink;
+  CK(hipMalloc(&in, nvec * 16));
+  CK(hipMalloc(&ticket, 256));
+  CK(hipMalloc(&sink, 256));
+  CK(hipMemset(in, 1, nvec * 16));
+  std::printf("tiles: 512-thread blocks that draw a ticket and read one tile of 1 GiB each (memset of the ticket included)\n");
+  run_tile_read<false, 0>(in, ticket, sink, 8192);
+  run_tile_read<true, 0>(in, ticket, sink, 8192);
+  run_tile_read<false, 0>(in, ticket, sink, 16384);
+  run_tile_read<true, 0>(in, ticket, sink, 16384);
+  run_tile_read<false, 16>(in, ticket, sink, (int)(nvec / (512 * 16)));
+  run_tile_read<true, 16>(in, ticket, sink, (int)(nvec / (512 * 16)));
+  run_tile_read<false, 12>(in, ticket, sink, (int)(nvec / (512 * 12)));
+  run_tile_read<true, 12>(in, ticket, sink, (int)(nvec / (512 * 12)));
+  run_tile_read<false, 8>(in, ticket, sink, (int)(nvec / (512 * 8)));
+  run_tile_read<true, 8>(in, ticket, sink, (int)(nvec / (512 * 8)));
+  CK(hipFree(in));
+  CK(hipFree(ticket));
+  CK(hipFree(sink));
+}
+
 int main(int argc, char** argv) {
   const char* which = argc > 1 ? argv[1] : "all";
   hipDeviceProp_t prop;
@@ -585,6 +655,7 @@ int main(int argc, char** argv) {
   if (all || std::strcmp(which, "scatter") == 0) section_scatter();
   if (all || std::strcmp(which, "lds") == 0) section_lds();
   if (all || std::strcmp(which, "latency") == 0) section_latency();
+  if (all || std::strcmp(which, "tiles") == 0) section_tiles();
   std::fflush(stdout);
   return 0;
 }
