@@ -238,7 +238,7 @@ int32_t ilgpu_hip_sort_check_device(ilgpu_hip_stream_t stream);
  *   LARGE_BLOCK_MIN_TILES_PER_CU  inputs of at least this many 1024-thread
  *     tiles per compute unit are sorted with 1024-thread blocks (longer runs
  *     per digit), smaller ones with 512-thread blocks (more blocks for fewer
- *     keys).  Default 10 for keys, 2 for pairs; 0 = always the large block,
+ *     keys).  Default 3 for keys, 2 for pairs; 0 = always the large block,
  *     INT32_MAX = never.
  *   ONE_TILE_KERNEL  inputs of at most one 512-thread tile (18432 keys of up
  *     to 4 bytes, fewer for wider keys and for pairs) are sorted by one block
