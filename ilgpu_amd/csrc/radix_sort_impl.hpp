@@ -380,11 +380,13 @@ __global__ __launch_bounds__(kHistBlock) void sort_histogram_kernel(
     run_key_count = 0u;
   };
   auto flush_half_run = [&]() {  // run_half: ordered bits above the lower half
-    if ((threadIdx.x & (kWaveSize - 1)) == 0 && run_half_count != 0u) {
+    if constexpr (sizeof(K) >= 2) {  // a 1-byte key has no upper half of whole digits
+      if ((threadIdx.x & (kWaveSize - 1)) == 0 && run_half_count != 0u) {
 #pragma unroll
-      for (int p = (int)sizeof(K) / 2; p < (int)sizeof(K); ++p)
-        atomicAdd(&s_hist[((p * kRadix + ((uint32_t)(run_half >> (8 * p - kHalfBits)) & (kRadix - 1))) << replica_shift) + replica],
-                  run_half_count);
+        for (int p = (int)sizeof(K) / 2; p < (int)sizeof(K); ++p)
+          atomicAdd(&s_hist[((p * kRadix + ((uint32_t)(run_half >> (8 * p - kHalfBits)) & (kRadix - 1))) << replica_shift) + replica],
+                    run_half_count);
+      }
     }
     run_half_count = 0u;
   };
@@ -1028,9 +1030,9 @@ void onesweep_kernel(
   // A grid of as many blocks as there are tiles (a short input) needs no
   // tickets (ticket == nullptr): block b takes tile b and is done, which saves
   // a pass two round trips to the ticket, one of them only to learn that
-  // there is nothing left.  Blocks are dispatched in index order, so a tile's
-  // predecessors have started; should they not be running, the bounded
-  // look-back covers that as it does with tickets.
+  // there is nothing left.  Blocks start in index order in practice, so a
+  // tile's predecessors are running; where they are not, the bounded look-back
+  // covers that as it does with tickets.
   for (int round = 0;; ++round) {
     int tile;
     if (ticket == nullptr) {
@@ -2309,8 +2311,8 @@ int32_t launch_sized(hipStream_t stream, const SortArgs& a) {
     rc = launch_passes<KEY_BYTES, VALUE_BYTES, kSortBlock>(stream, a, L, base, xf, cus);
   if (rc != ILGPU_HIP_SUCCESS) return rc;
   {
-    // Mostly there is nothing to copy and every block returns at once: a
-    // short input gets a grid that is dispatched quickly (16 keys per thread).
+    // Mostly there is nothing to copy and every block returns at once; 16
+    // keys per thread are few enough blocks for that and enough for the copy.
     int64_t blocks = div_up(a.n, 256 * 16);
     if (blocks > (int64_t)cus * 8) blocks = (int64_t)cus * 8;
     ProfileScope scope(stream, "sort_finish");
