@@ -29,6 +29,18 @@ def test_library_exports_every_declared_symbol():
     assert sorted(capi.EXPORTS) == names
 
 
+def test_binding_constants_are_the_headers():
+    # every enumerator of the header has the same value under the same name
+    # (without the ILGPU_HIP_ prefix) in the ctypes binding
+    header = open(HEADER).read()
+    enumerators = re.findall(r"\b(ILGPU_HIP_[A-Z0-9_]+)\s*=\s*(-?\d+)", header)
+    assert len(enumerators) >= 39
+    for name, value in enumerators:
+        short = name[len("ILGPU_HIP_"):]
+        assert hasattr(capi, short), name
+        assert getattr(capi, short) == int(value), name
+
+
 def test_version_and_status_strings():
     assert capi.lib().ilgpu_hip_version() == 100
     for status in range(6):
