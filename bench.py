@@ -46,6 +46,9 @@ def parse_args():
                    help="skip the CPU baseline")
     p.add_argument("--cpu-log2n", type=int, default=27,
                    help="log2 of the CPU baseline sample size")
+    p.add_argument("--short-sorts", action="store_true",
+                   help="instead of the benchmark: sorts of 2^15 to 2^23 keys with and "
+                        "without short tiles, one JSON line")
     return p.parse_args()
 
 
@@ -74,6 +77,40 @@ class Timer:
         wall = time.perf_counter() - wall0
         ms = [s.elapsed_time(e) for s, e in zip(starts, stops)]
         return ms, wall
+
+
+def short_sorts(torch, capi, datagen, timer, wrap, steps, warmup):
+    """Whole sorts of short inputs (keys without values) in the tile class they
+    take by default against full tiles (the library's test hook switches the
+    short classes off): median ms per sort, one JSON line."""
+    rows = {}
+    for name, dtype, sizes in (
+            ("u32", np.uint32, [1 << 15, 1 << 16, 1 << 17, 1 << 18, 1 << 19, 1 << 20, 1 << 21,
+                                3 << 20, 1 << 22, 5 << 20, 1 << 23]),
+            ("u64", np.uint64, [1 << 15, 1 << 16, 1 << 17, 1 << 18, 1 << 19, 1 << 20])):
+        for m in sizes:
+            if dtype == np.uint32:
+                part = datagen.uniform_u32_torch(m)
+            else:
+                part = datagen.splitmix64_torch(m)
+            wk = torch.empty_like(part)
+            kv = wrap(wk, dtype)
+            tp = capi.temp_buffer(capi.radix_sort_temp_bytes(m, dtype))
+            entry = {}
+            for label, limit in (("full_tiles_ms", 0), ("default_ms", -1)):
+                capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, limit)
+                ms, _ = timer.run(lambda: wk.copy_(part), lambda: capi.radix_sort_keys(kv, tp),
+                                  steps, warmup)
+                entry[label] = round(float(np.median(ms)), 4)
+            capi.sort_set_parameter(capi.SORT_PARAM_SHORT_TILE_MAX_TILES, -1)
+            # unsigned order through signed compares: low 32 bits widened, or
+            # the 64 bits with the sign bit flipped
+            srt = wk.to(torch.int64) & 0xFFFFFFFF if dtype == np.uint32 else wk ^ (-1 << 63)
+            entry["sorted"] = bool((srt[1:] >= srt[:-1]).all().item())
+            rows[f"{name}_{m}"] = entry
+            log(f"[bench] short sort {name} n={m}: full tiles {entry['full_tiles_ms']} ms, "
+                f"default {entry['default_ms']} ms")
+    print(json.dumps({"short_sorts": rows}))
 
 
 def kernel_stats(capi, name):
@@ -157,6 +194,10 @@ def main():
         """A DeviceArray over the memory of a torch tensor."""
         b = t.view(torch.uint8).reshape(-1)
         return D(b.numel() // np.dtype(dtype).itemsize, dtype, _bytes=b)
+
+    if args.short_sorts:
+        short_sorts(torch, capi, datagen, timer, wrap, max(K, 40), max(W, 5))
+        return
 
     # ------------------------------------------------------------ headline
     n = 1 << args.log2n
