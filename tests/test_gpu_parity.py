@@ -964,6 +964,48 @@ def test_sort_of_keys_that_agree_across_whole_waves(dtype):
         assert np.array_equal(gpu_sort(keys), np.sort(keys, kind="stable"))
 
 
+def test_sorts_of_random_shapes_under_random_test_hooks_match_oracle():
+    # 300 seeded cases: key type, length (one row to a few hundred tiles), key
+    # distribution (full range, a handful of values, constant), direction, keys
+    # or pairs, and every test hook that picks a code path (block size, one-tile
+    # kernel, short-tile limit, look-back bound) drawn at random.
+    rng = np.random.default_rng(20240607)
+    value_types = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}
+    for case in range(300):
+        dtype = ALL_KEY_DTYPES[int(rng.integers(len(ALL_KEY_DTYPES)))]
+        dt = np.dtype(dtype)
+        n = int(rng.choice([rng.integers(1, 300), rng.integers(1, 40000),
+                            rng.integers(1, 400000)]))
+        spin = int(rng.choice([-1, -1, -1, 0])) if n <= 200000 else -1
+        hooks = {capi.SORT_PARAM_LARGE_BLOCK_MIN_TILES_PER_CU: int(rng.choice([-1, -1, 0, 2**31 - 1])),
+                 capi.SORT_PARAM_ONE_TILE_KERNEL: int(rng.choice([1, 1, 0])),
+                 capi.SORT_PARAM_SHORT_TILE_MAX_TILES: int(rng.choice([-1, -1, 0, 40, 300])),
+                 capi.SORT_PARAM_LOOKBACK_SPIN_LIMIT: spin}
+        for parameter, value in hooks.items():
+            capi.sort_set_parameter(parameter, value)
+        mode = int(rng.integers(0, 3))
+        if dt.kind == "f":
+            keys = random_float_bits(dtype, n, seed=case) if mode == 0 else \
+                rng.integers(-3, 4, n).astype(dtype)
+        elif mode == 0:
+            keys = random_ints(dtype, n, seed=case)
+        elif mode == 1:
+            keys = rng.integers(0, 6, n).astype(dtype)
+        else:
+            keys = np.full(n, rng.integers(0, 100), dtype=dtype)
+        descending = bool(rng.integers(0, 2))
+        pairs = bool(rng.integers(0, 2))
+        note("random sort case", case, dt.name, n, mode, descending, pairs, sorted(hooks.items()))
+        if pairs:
+            values = np.arange(n).astype(value_types[int(rng.choice([1, 2, 4, 8]))])
+            k, v = gpu_sort_pairs(keys, values, descending=descending)
+            ek, ev = O.radix_sort_pairs(keys, values, descending=descending)
+            assert bits_equal(k, ek) and np.array_equal(v, ev), case
+        else:
+            assert bits_equal(gpu_sort(keys, descending=descending),
+                              O.radix_sort(keys, descending=descending)), case
+
+
 @pytest.fixture
 def no_short_tiles():
     """Short inputs of keys take full tiles like pairs and longer inputs do."""
